@@ -100,6 +100,26 @@ uint64_t nt_engine_weight_bytes(nt_engine_t e);            /* the model's tensor
 uint64_t nt_engine_resident_weight_bytes(nt_engine_t e);   /* what they occupy in HBM now: GGUF bytes still resident + the decode repack + the unpack scratch */
 uint64_t nt_engine_repacked_bytes(nt_engine_t e);          /* of which the decode repack (tensors that did not fit stay on the raw path and are not counted) */
 int  nt_engine_max_context(nt_engine_t e);
+/* ---- model folders -----------------------------------------------------------------------------------------------------------------
+ * nt_engine_load(_ex) also takes a FOLDER with config.json + model.safetensors (dense bfloat16 weights); the model class is picked by the
+ * config's "architecture" from the families built into the library.  Options, before the load: "dtype" = "bfloat16" (default: bf16 matrix
+ * products with F32 sums; norms, rotations, attention scores and weights, routers and the residual stream in F32) | "float32" (everything in
+ * true F32); "slots" = sequences the cache holds at once.  A folder holds no tokenizer: nt_engine_generate_tokens and nt_engine_forward work
+ * on ids (nt_engine_forward uses slot 0, re-based at start_pos); nt_engine_generate and the GGUF path's other entry points return an error.
+ * A sequence owns one slot of the cache from acquire to release (a released slot is handed out again as it is); nt_engine_seq_forward appends
+ * n tokens to it -- a whole prompt, a portion of any size, one decoded token -- and copies the logits of the places want[0..n_want) (ascending
+ * indices into these n tokens) to logits_out [n_want][vocab].  Logits of a position do not depend on how its sequence was cut into calls, beyond
+ * rounding.  nt_engine_seq_capture(1): the next forwards keep the residual stream after every layer run, nt_engine_seq_copy_capture copies the
+ * last call's [nt_engine_layer_runs][n][hidden] (parity instrumentation). */
+int  nt_engine_is_sequence_model(nt_engine_t e);
+int  nt_engine_layer_runs(nt_engine_t e);
+int  nt_engine_seq_acquire(nt_engine_t e);                     /* slot id >= 0, or negative */
+int  nt_engine_seq_release(nt_engine_t e, int slot);
+int  nt_engine_seq_length(nt_engine_t e, int slot);
+int  nt_engine_seq_truncate(nt_engine_t e, int slot, int length);
+int  nt_engine_seq_forward(nt_engine_t e, int slot, const int* tokens, int n, const int* want, int n_want, float* logits_out);
+int  nt_engine_seq_capture(nt_engine_t e, int on);
+int  nt_engine_seq_copy_capture(nt_engine_t e, float* out);
 /* which form the fused decode step takes at the current position: "fused (5 launches/layer)", or (EXPERIMENTS=1 builds with the
  * "persistent" option on) "persistent (...)" */
 const char* nt_engine_decode_path(nt_engine_t e);

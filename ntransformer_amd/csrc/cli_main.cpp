@@ -4,6 +4,8 @@
 #include <cstdio>
 #include <cstring>
 #include <string>
+#include <vector>
+#include <cstdlib>
 #include "engine/engine.h"
 #include "../../include/ntk_engine.h"
 
@@ -11,7 +13,9 @@ static void usage(const char* prog) {
     fprintf(stderr,
             "NTransformer (MI355X-native) - quantized LLM decode engine\n\n"
             "Usage: %s [options] -m <model.gguf>\n\nOptions:\n"
-            "  -m, --model <path>       Path to GGUF model file (required unless --synthetic)\n"
+            "  -m, --model <path>       Path to GGUF model file, or a model folder (config.json + model.safetensors)\n"
+            "  --tokens <id,id,...>     Prompt as token ids; prints the generated ids (model folders hold no tokenizer)\n"
+            "  --dtype <bfloat16|float32>  Model folders: bf16 matrix products (default) or everything in F32\n"
             "  -p, --prompt <text>      Prompt text (default: interactive mode)\n"
             "  -n, --n-tokens <int>     Max tokens to generate (default: 256)\n"
             "  -t, --temperature <float> Temperature (default: 0.7)\n"
@@ -36,7 +40,7 @@ static void usage(const char* prog) {
 }
 
 int main(int argc, char** argv) {
-    std::string model_path, prompt, synthetic;
+    std::string model_path, prompt, synthetic, token_list;
     int max_context = 4096;
     bool benchmark = false, chat = false;
     nt::GenerateConfig cfg;
@@ -72,6 +76,12 @@ int main(int argc, char** argv) {
         else if (a == "--no-batched-prefill") engine.options().batched_prefill = false;
         else if (a == "--no-graph") engine.options().graph = false;
         else if (a == "--synthetic") { if (auto v = val()) synthetic = v; }
+        else if (a == "--tokens") { if (auto v = val()) token_list = v; }
+        else if (a == "--dtype") {
+            const char* v = val();
+            if (!v || (strcmp(v, "bfloat16") && strcmp(v, "float32"))) { fprintf(stderr, "--dtype takes bfloat16 or float32\n"); return 1; }
+            engine.options().float32 = !strcmp(v, "float32");
+        }
         else if (a == "--streaming") noop(a.c_str(), "weights are fully resident on MI355X");
         else if (a == "--self-spec") noop(a.c_str(), "plain decode runs (same tokens under greedy decoding, no draft pass)");
         else if (a == "--draft-model" || a == "--draft-k") { (void)val(); noop(a.c_str(), "plain decode runs (same tokens under greedy decoding, no draft model is loaded)"); }
@@ -96,6 +106,23 @@ int main(int argc, char** argv) {
     }
     if (st != NTK_OK) { fprintf(stderr, "Failed to load model: %s (%s)\n", model_path.c_str(), engine.error().c_str()); return 1; }
 
+    if (!token_list.empty() || engine.is_sequence_model()) {
+        // generation on ids: the path of a model folder (and of a GGUF model when --tokens is given)
+        std::vector<int> ids, out;
+        for (size_t at = 0; at < token_list.size();) {
+            const size_t c = token_list.find(',', at);
+            ids.push_back(atoi(token_list.substr(at, c == std::string::npos ? std::string::npos : c - at).c_str()));
+            if (c == std::string::npos) break;
+            at = c + 1;
+        }
+        if (ids.empty()) { fprintf(stderr, "Error: a model folder is prompted with --tokens <id,id,...>\n"); return 1; }
+        const int rc = engine.generate_tokens(ids, cfg, out, true);
+        if (rc != NTK_OK) { fprintf(stderr, "Generation failed: %s\n", engine.error().c_str()); return 1; }
+        for (size_t i = 0; i < out.size(); ++i) printf("%s%d", i ? "," : "", out[i]);
+        printf("\n");
+        engine.print_stats(engine.last_stats());
+        return 0;
+    }
     if (benchmark) engine.benchmark(prompt.empty() ? "The meaning of life is" : prompt, cfg.max_tokens);
     else if (chat || prompt.empty()) engine.chat(cfg);
     else engine.generate(prompt, cfg);

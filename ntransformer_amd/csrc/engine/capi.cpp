@@ -13,6 +13,8 @@ using nt::Engine;
 
 namespace {
 Engine* E(nt_engine_t e) { return static_cast<Engine*>(e); }
+// loaded from a GGUF file (nt::Model): what the entry points of the Llama path need; a model folder answers them with an error / zero
+bool GGUF(nt_engine_t e) { return E(e)->loaded() && !E(e)->is_sequence_model(); }
 nt::SynthSpec to_spec(const nt_synth_spec& s) {
     nt::SynthSpec o;
     o.hidden = s.hidden; o.inter = s.inter; o.layers = s.layers; o.heads = s.heads; o.kv_heads = s.kv_heads;
@@ -54,6 +56,14 @@ int nt_engine_set_option(nt_engine_t e, const char* key, const char* value) {
     if (!e || !key || !value) return NTK_E_NULL;
     const bool on = atoi(value) != 0;
     const std::string k = key;
+    if (k == "dtype") {   // model folders, before the load: "bfloat16" (default) | "float32"
+        const std::string v = value;
+        if (v != "bfloat16" && v != "float32") return NTK_E_DTYPE;
+        E(e)->options().float32 = v == "float32";
+        return NTK_OK;
+    }
+    if (k == "slots") { if (atoi(value) < 1) return NTK_E_SHAPE; E(e)->options().slots = atoi(value); return NTK_OK; }
+    if (E(e)->is_sequence_model()) return NTK_E_SHAPE;   // the remaining options belong to the GGUF path
     if (k == "fused") E(e)->options().fused = on;
     else if (k == "graph") E(e)->options().graph = on;
     else if (k == "batched_prefill") { E(e)->options().batched_prefill = on; E(e)->model().set_batched_prefill(on); }
@@ -94,10 +104,29 @@ char* nt_engine_generate(nt_engine_t e, const char* prompt, int max_tokens, floa
 }
 void nt_free(char* p) { free(p); }
 
-int nt_engine_vocab_size(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->model().config().vocab_size : -1; }
-int nt_engine_n_layers(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->model().config().n_layers : -1; }
-int nt_engine_hidden_size(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->model().config().hidden_size : -1; }
-int nt_engine_max_context(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->model().config().max_seq_len : -1; }
+int nt_engine_vocab_size(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->vocab_size() : -1; }
+int nt_engine_n_layers(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->n_layers() : -1; }
+int nt_engine_hidden_size(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->hidden_size() : -1; }
+int nt_engine_max_context(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->max_context() : -1; }
+
+// ---- model folders: the slot cache and the step, as the trace runner and the generation loop use them
+static nt::SequenceModel* SEQ(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->sequence_model() : nullptr; }
+int nt_engine_is_sequence_model(nt_engine_t e) { return SEQ(e) ? 1 : 0; }
+int nt_engine_layer_runs(nt_engine_t e) { return SEQ(e) ? SEQ(e)->info().n_layer_runs : -1; }
+int nt_engine_seq_acquire(nt_engine_t e) { return SEQ(e) ? SEQ(e)->acquire_slot() : NTK_E_NULL; }
+int nt_engine_seq_release(nt_engine_t e, int slot) { return SEQ(e) ? SEQ(e)->release_slot(slot) : NTK_E_NULL; }
+int nt_engine_seq_length(nt_engine_t e, int slot) { return SEQ(e) ? SEQ(e)->slot_length(slot) : NTK_E_NULL; }
+int nt_engine_seq_truncate(nt_engine_t e, int slot, int length) { return SEQ(e) ? SEQ(e)->truncate_slot(slot, length) : NTK_E_NULL; }
+int nt_engine_seq_forward(nt_engine_t e, int slot, const int* tokens, int n, const int* want, int n_want, float* logits_out) {
+    if (!SEQ(e)) return NTK_E_NULL;
+    if (!tokens || (n_want > 0 && (!want || !logits_out))) return NTK_E_NULL;
+    try {
+        if (!SEQ(e)->forward(slot, tokens, n, want, n_want)) return NTK_E_LAUNCH;
+        return n_want > 0 ? SEQ(e)->copy_logits(logits_out, n_want) : SEQ(e)->sync();
+    } catch (...) { return NTK_E_NOMEM; }
+}
+int nt_engine_seq_capture(nt_engine_t e, int on) { return SEQ(e) ? SEQ(e)->set_capture(on != 0) : NTK_E_NULL; }
+int nt_engine_seq_copy_capture(nt_engine_t e, float* out) { return SEQ(e) && out ? SEQ(e)->copy_capture(out) : NTK_E_NULL; }
 
 int nt_engine_generate_tokens(nt_engine_t e, const int* prompt, int n_prompt, const nt_gen_params* p, int* out, int out_cap) {
     if (!e || !prompt || !p || (!out && out_cap > 0)) return NTK_E_NULL;
@@ -126,13 +155,22 @@ int nt_engine_last_stats(nt_engine_t e, nt_stats* o) {
 int nt_engine_forward(nt_engine_t e, const int* tokens, int n, int start_pos, float* logits_out) {
     if (!e || !tokens || !logits_out) return NTK_E_NULL;
     if (!E(e)->loaded()) return NTK_E_NULL;
+    if (nt::SequenceModel* m = E(e)->sequence_model()) {   // slot 0, re-based at start_pos
+        if (m->slot_length(0) < 0 && m->acquire_slot() != 0) return NTK_E_SHAPE;
+        if (start_pos > m->slot_length(0)) return NTK_E_SHAPE;
+        int rc = m->truncate_slot(0, start_pos);
+        if (rc != NTK_OK) return rc;
+        const int last = n - 1;
+        if (n <= 0 || !m->forward(0, tokens, n, &last, 1)) return NTK_E_LAUNCH;
+        return m->copy_logits(logits_out, 1);
+    }
     float* d = E(e)->model().forward(tokens, n, start_pos);
     if (!d) return NTK_E_LAUNCH;
     return E(e)->model().copy_logits(logits_out);
 }
 
 int nt_engine_decode_fused(nt_engine_t e, int token, int pos, int use_graph, float* logits_out) {
-    if (!e || !logits_out || !E(e)->loaded()) return NTK_E_NULL;
+    if (!e || !logits_out || !GGUF(e)) return NTK_E_NULL;
     nt::Model& m = E(e)->model();
     if (pos < 0 || pos >= m.config().max_seq_len) return NTK_E_SHAPE;
     m.set_device_pos(pos);
@@ -147,44 +185,44 @@ int nt_engine_decode_fused(nt_engine_t e, int token, int pos, int use_graph, flo
 
 int nt_engine_debug_run_layers(nt_engine_t e, const float* hidden_in, int n_tokens, int start_pos, int first_layer, int n_layers, int mode,
                                float* hidden_out) {
-    if (!e || !E(e)->loaded()) return NTK_E_NULL;
+    if (!e || !GGUF(e)) return NTK_E_NULL;
     return E(e)->model().debug_run_layers(hidden_in, n_tokens, start_pos, first_layer, n_layers, mode, hidden_out);
 }
 int nt_engine_debug_kv_read(nt_engine_t e, int layer, int pos0, int n, uint16_t* k_out, uint16_t* v_out) {
-    if (!e || !E(e)->loaded()) return NTK_E_NULL;
+    if (!e || !GGUF(e)) return NTK_E_NULL;
     return E(e)->model().debug_kv(layer, pos0, n, k_out, v_out, false);
 }
 int nt_engine_debug_kv_write(nt_engine_t e, int layer, int pos0, int n, const uint16_t* k, const uint16_t* v) {
-    if (!e || !E(e)->loaded()) return NTK_E_NULL;
+    if (!e || !GGUF(e)) return NTK_E_NULL;
     return E(e)->model().debug_kv(layer, pos0, n, const_cast<uint16_t*>(k), const_cast<uint16_t*>(v), true);
 }
 
-void* nt_engine_persistent_plan(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->model().persistent_plan() : nullptr; }
-int nt_engine_persistent_kind(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->model().persistent_kind() : 0; }
-const char* nt_engine_decode_path(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->model().decode_path() : ""; }
+void* nt_engine_persistent_plan(nt_engine_t e) { return e && GGUF(e) ? E(e)->model().persistent_plan() : nullptr; }
+int nt_engine_persistent_kind(nt_engine_t e) { return e && GGUF(e) ? E(e)->model().persistent_kind() : 0; }
+const char* nt_engine_decode_path(nt_engine_t e) { return e && GGUF(e) ? E(e)->model().decode_path() : ""; }
 
 // ---- tensor parallelism (one engine per rank; csrc/tp.hip) ---------------------------------------------------------------
 int nt_engine_tp_configure(nt_engine_t e, int rank, int world) { return e ? E(e)->model().tp_configure(rank, world) : NTK_E_NULL; }
 int nt_engine_tp_export(nt_engine_t e, void* handle64, void** raw) {
-    if (!e || !E(e)->loaded()) return NTK_E_NULL;
+    if (!e || !GGUF(e)) return NTK_E_NULL;
     return E(e)->model().tp_export(handle64, raw);
 }
 int nt_engine_tp_connect(nt_engine_t e, const void* handles, void* const* raws) {
-    if (!e || !E(e)->loaded()) return NTK_E_NULL;
+    if (!e || !GGUF(e)) return NTK_E_NULL;
     return E(e)->model().tp_connect(handles, raws);
 }
-unsigned nt_engine_tp_error(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->model().tp_error() : 0u; }
+unsigned nt_engine_tp_error(nt_engine_t e) { return e && GGUF(e) ? E(e)->model().tp_error() : 0u; }
 int nt_tp_slice_columns(void* dst, const void* src, int dtype, int64_t out_features, int64_t in_features, int rank, int world) {
     return nt::Model::slice_columns(dst, src, dtype, out_features, in_features, rank, world);   // host only
 }
 
 int nt_engine_decode_greedy_steps(nt_engine_t e, int token, int pos, int n, int* out) {
-    if (!e || !E(e)->loaded()) return NTK_E_NULL;
+    if (!e || !GGUF(e)) return NTK_E_NULL;
     return E(e)->decode_greedy_steps(token, pos, n, out);
 }
 
 int nt_engine_profile_token(nt_engine_t e, int token, int pos, int coarse, float* ms4, int* calls4) {
-    if (!e || !ms4 || !calls4 || !E(e)->loaded()) return NTK_E_NULL;
+    if (!e || !ms4 || !calls4 || !GGUF(e)) return NTK_E_NULL;
     nt::Model& m = E(e)->model();
     if (pos < 0 || pos >= m.config().max_seq_len) return NTK_E_SHAPE;
     m.set_device_pos(pos);
@@ -194,14 +232,14 @@ int nt_engine_profile_token(nt_engine_t e, int token, int pos, int coarse, float
 }
 
 int nt_engine_tokenize(nt_engine_t e, const char* text, int add_bos, int* out, int cap) {
-    if (!e || !text || !E(e)->loaded()) return NTK_E_NULL;
+    if (!e || !text || !GGUF(e)) return NTK_E_NULL;
     const std::vector<int> ids = E(e)->tokenizer().encode(text, add_bos != 0);
     for (int i = 0; i < (int)ids.size() && i < cap; ++i) out[i] = ids[i];
     return (int)ids.size();
 }
 
 int nt_engine_detokenize(nt_engine_t e, const int* ids, int n, char* out, int cap) {
-    if (!e || !ids || !E(e)->loaded()) return NTK_E_NULL;
+    if (!e || !ids || !GGUF(e)) return NTK_E_NULL;
     const std::string s = E(e)->tokenizer().decode(std::vector<int>(ids, ids + n));
     if (out && cap > 0) {
         const size_t k = std::min<size_t>(s.size(), (size_t)cap - 1);
@@ -211,10 +249,13 @@ int nt_engine_detokenize(nt_engine_t e, const int* ids, int n, char* out, int ca
     return (int)s.size();
 }
 
-uint64_t nt_engine_bytes_per_token(nt_engine_t e, int pos) { return e && E(e)->loaded() ? E(e)->model().bytes_per_token(pos) : 0; }
-uint64_t nt_engine_weight_bytes(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->model().weight_bytes() : 0; }
-uint64_t nt_engine_resident_weight_bytes(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->model().resident_weight_bytes() : 0; }
-uint64_t nt_engine_repacked_bytes(nt_engine_t e) { return e && E(e)->loaded() ? E(e)->model().repack_bytes() : 0; }
+uint64_t nt_engine_bytes_per_token(nt_engine_t e, int pos) { return e && GGUF(e) ? E(e)->model().bytes_per_token(pos) : 0; }
+uint64_t nt_engine_weight_bytes(nt_engine_t e) {
+    if (e && E(e)->loaded() && E(e)->is_sequence_model()) return E(e)->sequence_model()->weight_bytes();
+    return e && GGUF(e) ? E(e)->model().weight_bytes() : 0;
+}
+uint64_t nt_engine_resident_weight_bytes(nt_engine_t e) { return e && GGUF(e) ? E(e)->model().resident_weight_bytes() : 0; }
+uint64_t nt_engine_repacked_bytes(nt_engine_t e) { return e && GGUF(e) ? E(e)->model().repack_bytes() : 0; }
 
 int nt_synth_write_gguf(const char* path, const nt_synth_spec* spec, int nthreads) {
     if (!path || !spec) return NTK_E_NULL;

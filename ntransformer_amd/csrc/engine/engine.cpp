@@ -1,5 +1,6 @@
 // engine/engine.cpp -- see engine.h
 #include "engine.h"
+#include "safetensors.h"
 #include "../../../include/ntk_engine.h"
 
 #include <chrono>
@@ -14,6 +15,17 @@ static float ms_since(Clock::time_point t0) { return std::chrono::duration<float
 
 int Engine::load(const std::string& path, int max_context) {
     loaded_ = false;
+    seq_.reset();
+    if (ModelFolder::looks_like(path)) {
+        SeqLoadOptions o;
+        o.max_context = max_context;
+        o.slots = opt_.slots > 0 ? opt_.slots : 1;
+        o.float32 = opt_.float32;
+        seq_ = open_model(path, o, &err_);
+        if (!seq_) return NTK_E_FORMAT;
+        loaded_ = true;
+        return NTK_OK;
+    }
     const int st = model_.load(path, max_context);
     if (st != NTK_OK) { err_ = model_.error(); return st; }
     tok_.init(model_.vocab(), model_.config().bos_token_id, model_.config().eos_token_id);   // engine.cpp:21
@@ -23,6 +35,7 @@ int Engine::load(const std::string& path, int max_context) {
 
 int Engine::load_synthetic(const SynthSpec& spec, int max_context) {
     loaded_ = false;
+    seq_.reset();
     int nt = opt_.synth_threads > 0 ? opt_.synth_threads : (int)std::thread::hardware_concurrency();
     const int st = model_.load_synthetic(spec, max_context, nt > 0 ? nt : 8);
     if (st != NTK_OK) { err_ = model_.error(); return st; }
@@ -34,6 +47,8 @@ int Engine::load_synthetic(const SynthSpec& spec, int max_context) {
 int Engine::load_shared(Engine& src, int max_context) {
     loaded_ = false;
     if (!src.loaded_) { err_ = "load_shared: the source engine is not loaded"; return NTK_E_NULL; }
+    if (src.seq_) { err_ = "load_shared: a model folder serves several sequences from the slots of ONE engine (option \"slots\")"; return NTK_E_SHAPE; }
+    seq_.reset();
     const int st = model_.share_weights(src.model_, max_context);
     if (st != NTK_OK) { err_ = model_.error(); return st; }
     tok_.init(model_.vocab(), model_.config().bos_token_id, model_.config().eos_token_id);
@@ -49,6 +64,7 @@ int Engine::run(std::vector<int>& tokens, const GenerateConfig& cfg, std::string
     stats_ = Stats();
     if (!loaded_) { err_ = "model not loaded"; return NTK_E_NULL; }
     if (tokens.empty()) { err_ = "empty prompt"; return NTK_E_SHAPE; }
+    if (seq_) return run_sequence(tokens, cfg, cb, stop_at_eos);
     Sampler sampler;
     SamplerConfig sc;
     sc.temperature = cfg.temperature; sc.top_k = cfg.top_k; sc.top_p = cfg.top_p;
@@ -148,8 +164,55 @@ int Engine::run(std::vector<int>& tokens, const GenerateConfig& cfg, std::string
     return rc;
 }
 
+// The generation loop of a model folder: one slot of the family's cache, the prompt in one forward (the family cuts it into its own passes), then
+// one token per forward; the reference's sampler and repeat penalty on the host (engine.cpp:66-134).  Tokens are ids: a folder has no tokenizer, so the
+// callback gets an empty piece and the id.
+int Engine::run_sequence(std::vector<int>& tokens, const GenerateConfig& cfg, TokenCallback cb, bool stop_at_eos) {
+    Sampler sampler;
+    SamplerConfig sc;
+    sc.temperature = cfg.temperature; sc.top_k = cfg.top_k; sc.top_p = cfg.top_p;
+    sc.repeat_penalty = cfg.repeat_penalty; sc.repeat_window = cfg.repeat_window; sc.seed = cfg.seed;
+    sampler.init(sc);
+    const int V = seq_->info().vocab, eos = seq_->info().eos;
+    stats_.prompt_tokens = (int)tokens.size();
+    const int slot = seq_->acquire_slot();
+    if (slot < 0) { err_ = "every slot of the cache is taken"; return NTK_E_NOMEM; }
+    int rc = NTK_OK;
+    std::vector<float> host((size_t)V);
+    auto step = [&](const int* t, int n) -> int {
+        const int last = n - 1;
+        if (!seq_->forward(slot, t, n, &last, 1)) { err_ = seq_->error(); return NTK_E_LAUNCH; }
+        return seq_->copy_logits(host.data(), 1);
+    };
+    auto t0 = Clock::now();
+    rc = step(tokens.data(), (int)tokens.size());
+    stats_.prefill_ms = ms_since(t0);
+    if (rc == NTK_OK) {
+        sampler.apply_repeat_penalty(host.data(), V, tokens);
+        int next = sampler.sample(host.data(), V);
+        tokens.push_back(next);
+        bool go = !cb || cb(std::string(), next);
+        auto d0 = Clock::now();
+        for (int i = 1; go && i < cfg.max_tokens; ++i) {
+            if (stop_at_eos && eos >= 0 && next == eos) break;
+            if (seq_->slot_length(slot) >= seq_->info().max_context) break;
+            if ((rc = step(&next, 1)) != NTK_OK) break;
+            sampler.apply_repeat_penalty(host.data(), V, tokens);
+            next = sampler.sample(host.data(), V);
+            tokens.push_back(next);
+            ++stats_.gen_tokens;
+            if (cb && !cb(std::string(), next)) break;
+        }
+        stats_.decode_ms = ms_since(d0);
+    }
+    seq_->release_slot(slot);
+    if (rc != NTK_OK && err_.empty()) err_ = std::string("decode failed: ") + ntk_status_string(rc);
+    return rc;
+}
+
 int Engine::decode_greedy_steps(int token, int pos, int n, int* out) {
     if (!loaded_) return NTK_E_NULL;
+    if (seq_) { err_ = "decode_greedy_steps: a model folder decodes through generate_tokens / the nt_engine_seq_* calls"; return NTK_E_SHAPE; }
     if (pos < 0 || pos + n > model_.config().max_seq_len) return NTK_E_SHAPE;
     int next = token;
     if (opt_.fused) {
@@ -182,6 +245,7 @@ int Engine::decode_greedy_steps(int token, int pos, int n, int* out) {
 }
 
 std::string Engine::generate(const std::string& prompt, const GenerateConfig& cfg, TokenCallback cb) {
+    if (seq_) { err_ = "a model folder has no tokenizer: generate on token ids (generate_tokens, --tokens)"; return std::string(); }
     std::vector<int> tokens = tok_.encode(prompt, true);
     std::string out;
     run(tokens, cfg, &out, cb, cfg.verbose, true);
@@ -199,6 +263,7 @@ int Engine::generate_tokens(const std::vector<int>& prompt, const GenerateConfig
 }
 
 void Engine::chat(const GenerateConfig& cfg) {   // engine.cpp:545-570: stateless turns
+    if (seq_) { fprintf(stderr, "chat needs a tokenizer; a model folder has none (use --tokens)\n"); return; }
     fprintf(stdout, "NTransformer Chat (type 'quit' to exit)\nModel: %s (%d params)\n---\n", model_.config().model_name.c_str(),
             model_.config().n_layers);
     std::string line;

@@ -8,6 +8,7 @@
 #include <vector>
 #include "model.h"
 #include "sampler.h"
+#include "sequence_model.h"
 #include "tokenizer.h"
 
 namespace nt {
@@ -41,6 +42,9 @@ struct EngineOptions {
     bool device_sampling = true;  // greedy argmax on the device when temperature <= 0 and repeat_penalty <= 1
     bool persistent = false;      // short contexts: the whole token in one persistent launch (decode_persistent.hip)
     int synth_threads = 0;        // 0 = hardware concurrency
+    // model folders (config.json + model.safetensors, engine/sequence_model.h); read by load()
+    bool float32 = false;         // every product in true F32 instead of bf16 products with F32 sums
+    int slots = 1;                // sequences the cache holds at once (generate uses one; the nt_engine_seq_* calls may hold the others)
 };
 
 class Engine {
@@ -58,6 +62,15 @@ public:
     void benchmark(const std::string& prompt, int n_tokens);
     void print_stats(const Stats& st) const;
 
+    // A model FOLDER loads through the family registry (engine/sequence_model.h) instead of nt::Model; generation then runs on token ids
+    // (a folder holds no tokenizer), through the same sampler, one slot of the family's cache per generation.
+    bool is_sequence_model() const { return seq_ != nullptr; }
+    SequenceModel* sequence_model() { return seq_.get(); }
+    int vocab_size() const { return seq_ ? seq_->info().vocab : model_.config().vocab_size; }
+    int n_layers() const { return seq_ ? seq_->info().n_layers : model_.config().n_layers; }
+    int hidden_size() const { return seq_ ? seq_->info().width : model_.config().hidden_size; }
+    int max_context() const { return seq_ ? seq_->info().max_context : model_.config().max_seq_len; }
+
     Model& model() { return model_; }
     const Tokenizer& tokenizer() const { return tok_; }
     const Stats& last_stats() const { return stats_; }
@@ -67,6 +80,8 @@ public:
 
 private:
     int run(std::vector<int>& tokens, const GenerateConfig& cfg, std::string* text, TokenCallback cb, bool print, bool stop_at_eos);
+    int run_sequence(std::vector<int>& tokens, const GenerateConfig& cfg, TokenCallback cb, bool stop_at_eos);
+    std::unique_ptr<SequenceModel> seq_;
     Model model_;
     Tokenizer tok_;
     Stats stats_;

@@ -91,6 +91,14 @@ def _bind():
     L.nt_engine_debug_run_layers.argtypes = [vp, vp, i, i, i, i, i, vp]
     L.nt_engine_debug_kv_read.argtypes = [vp, i, i, i, vp, vp]
     L.nt_engine_debug_kv_write.argtypes = [vp, i, i, i, vp, vp]
+    for n in ("is_sequence_model", "layer_runs", "seq_acquire"):
+        getattr(L, "nt_engine_" + n).argtypes = [vp]
+    L.nt_engine_seq_release.argtypes = [vp, i]
+    L.nt_engine_seq_length.argtypes = [vp, i]
+    L.nt_engine_seq_truncate.argtypes = [vp, i, i]
+    L.nt_engine_seq_forward.argtypes = [vp, i, C.POINTER(i), i, C.POINTER(i), i, vp]
+    L.nt_engine_seq_capture.argtypes = [vp, i]
+    L.nt_engine_seq_copy_capture.argtypes = [vp, vp]
     L._engine_bound = True
     return L
 
@@ -158,7 +166,56 @@ class Engine:
         return int(self.L.nt_engine_tp_error(self.h))
 
     def set_option(self, key: str, value) -> None:
-        self._check(self.L.nt_engine_set_option(self.h, key.encode(), str(int(value)).encode()), "set_option " + key)
+        text = value if isinstance(value, str) else str(int(value))
+        self._check(self.L.nt_engine_set_option(self.h, key.encode(), text.encode()), "set_option " + key)
+
+    # ---- model folders (include/ntransformer.h: nt_engine_seq_*): one slot of the cache per live sequence ----
+    def load_folder(self, path: str, max_context: int = 4096, dtype: str = "bfloat16", slots: int = 1) -> None:
+        """a folder with config.json + model.safetensors; the model class comes from the config's architecture"""
+        self.set_option("dtype", dtype)
+        self.set_option("slots", slots)
+        self.load(path, max_context)
+
+    @property
+    def is_sequence_model(self) -> bool:
+        return bool(self.L.nt_engine_is_sequence_model(self.h))
+
+    @property
+    def layer_runs(self) -> int:
+        return self.L.nt_engine_layer_runs(self.h)
+
+    def seq_acquire(self) -> int:
+        s = self.L.nt_engine_seq_acquire(self.h)
+        if s < 0:
+            self._check(s, "seq_acquire")
+        return s
+
+    def seq_release(self, slot: int) -> None:
+        self._check(self.L.nt_engine_seq_release(self.h, slot), "seq_release")
+
+    def seq_length(self, slot: int) -> int:
+        return self.L.nt_engine_seq_length(self.h, slot)
+
+    def seq_truncate(self, slot: int, length: int) -> None:
+        self._check(self.L.nt_engine_seq_truncate(self.h, slot, length), "seq_truncate")
+
+    def seq_forward(self, slot: int, tokens: Sequence[int], want: Optional[Sequence[int]] = None) -> np.ndarray:
+        """append `tokens` to the slot; logits [len(want), vocab] of the places `want` (default: every token of this portion)"""
+        want = list(range(len(tokens))) if want is None else [int(w) for w in want]
+        out = np.empty((len(want), self.vocab_size), np.float32)
+        arr = (C.c_int * len(tokens))(*[int(t) for t in tokens])
+        warr = (C.c_int * max(len(want), 1))(*want)
+        self._check(self.L.nt_engine_seq_forward(self.h, slot, arr, len(tokens), warr, len(want), out.ctypes.data_as(C.c_void_p)), "seq_forward")
+        return out
+
+    def seq_capture(self, on: bool = True) -> None:
+        self._check(self.L.nt_engine_seq_capture(self.h, int(on)), "seq_capture")
+
+    def seq_captured(self, n_tokens: int) -> np.ndarray:
+        """the residual stream after every layer run of the last seq_forward: [layer runs, n_tokens, hidden]"""
+        out = np.empty((self.layer_runs, n_tokens, self.hidden_size), np.float32)
+        self._check(self.L.nt_engine_seq_copy_capture(self.h, out.ctypes.data_as(C.c_void_p)), "seq_copy_capture")
+        return out
 
     @property
     def vocab_size(self): return self.L.nt_engine_vocab_size(self.h)

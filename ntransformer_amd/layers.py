@@ -1,0 +1,208 @@
+"""Python view of include/ntk_layers.h: the operators of the layer-list model families, numpy in / numpy out (every call uploads its
+operands, launches on the library's compute stream and downloads the result -- for tests and micro-benchmarks, not a serving path).
+Weights are passed as float arrays and stored as bfloat16 (dtype="bfloat16", rounded to nearest even) or float32 on the device."""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional
+
+import numpy as np
+
+from . import _lib
+from ._lib import check
+from .ops import DeviceBuffer
+
+DT_F32, DT_BF16 = 0, 9
+
+
+class DenseDesc(C.Structure):
+    _fields_ = [("Y", C.c_void_p), ("ldy", C.c_int), ("X", C.c_void_p), ("ldx", C.c_int), ("W", C.c_void_p), ("wstride", C.c_longlong), ("wdtype", C.c_int),
+                ("offsets", C.c_void_p), ("G", C.c_int), ("rows", C.c_void_p), ("row_div", C.c_int), ("T", C.c_int), ("N", C.c_int), ("K", C.c_int),
+                ("accumulate", C.c_int)]
+
+
+class Rotary(C.Structure):
+    _fields_ = [("freq", C.c_void_p), ("mag", C.c_float), ("dims", C.c_int)]
+
+
+def _bind():
+    L = _lib.lib()
+    if getattr(L, "_layers_bound", False):
+        return L
+    vp, i, f, ll = C.c_void_p, C.c_int, C.c_float, C.c_longlong
+    L.ntk_dense.argtypes = [C.POINTER(DenseDesc), vp]
+    L.ntk_dense_linear.argtypes = [vp, i, vp, i, vp, i, i, i, i, i, vp]
+    L.ntk_embed_dense.argtypes = [vp, vp, i, vp, i, i, i, vp]
+    L.ntk_rmsnorm_offset.argtypes = [vp, vp, vp, vp, i, vp, i, i, i, f, f, vp]
+    L.ntk_concat_rows.argtypes = [vp, vp, vp, i, i, vp]
+    L.ntk_sigmoid_gate.argtypes = [vp, i, vp, i, i, i, vp]
+    L.ntk_rows_copy.argtypes = [vp, vp, ll, vp]
+    L.ntk_residual_add.argtypes = [vp, vp, vp, i, vp]
+    L.ntk_latent_prepare.argtypes = [vp, i, vp, i, vp, f, i, i, vp, i, i, i, C.POINTER(Rotary), i, i, vp]
+    L.ntk_latent_attention_scratch.argtypes = [i, i, i, i]
+    L.ntk_latent_attention_scratch.restype = C.c_size_t
+    L.ntk_latent_attention.argtypes = [vp, i, vp, i, vp, i, vp, i, vp, i, i, i, i, i, i, i, i, i, i, i, f, vp, vp]
+    L.ntk_latent_fold_query.argtypes = [vp, vp, i, vp, i, i, i, i, i, i, vp]
+    L.ntk_latent_unfold_value.argtypes = [vp, i, vp, vp, i, vp, i, i, i, i, i, vp]
+    L.ntk_moe_route.argtypes = [vp, vp, vp, vp, i, vp, vp, i, i, i, i, vp]
+    L.ntk_moe_group.argtypes = [vp, vp, vp, vp, i, i, i, vp]
+    L.ntk_clipped_glu.argtypes = [vp, vp, i, i, f, f, vp]
+    L.ntk_moe_combine.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, vp]
+    L._layers_bound = True
+    return L
+
+
+def to_bf16_bits(a: np.ndarray) -> np.ndarray:
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    u = u + 0x7FFF + ((u >> 16) & 1)
+    return (u >> 16).astype(np.uint16)
+
+
+def from_bf16_bits(b: np.ndarray) -> np.ndarray:
+    return (b.astype(np.uint32) << 16).view(np.float32)
+
+
+def weight_buffer(w: np.ndarray, dtype: str) -> tuple:
+    """(DeviceBuffer, NTK_DT_*) of a weight array in the given storage"""
+    if dtype == "bfloat16":
+        return DeviceBuffer.from_numpy(to_bf16_bits(w)), DT_BF16
+    if dtype == "float32":
+        return DeviceBuffer.from_numpy(np.ascontiguousarray(w, np.float32)), DT_F32
+    raise ValueError(dtype)
+
+
+def _f(a) -> DeviceBuffer:
+    return DeviceBuffer.from_numpy(np.ascontiguousarray(a, np.float32))
+
+
+def _i(a) -> DeviceBuffer:
+    return DeviceBuffer.from_numpy(np.ascontiguousarray(a, np.int32))
+
+
+def dense(x: np.ndarray, w: np.ndarray, dtype: str = "float32", offsets=None, rows=None, row_div: int = 1, n_rows: Optional[int] = None,
+          y0: Optional[np.ndarray] = None) -> np.ndarray:
+    """y[r] = x[src(r)] . w[g(r)]^T; w [N, K] or a stack [G, N, K] with `offsets` [G + 1]; rows: source row per output row (divided by row_div);
+    y0: start values to accumulate onto."""
+    L = _bind()
+    w = np.asarray(w)
+    stacked = w.ndim == 3
+    N, K = w.shape[-2], w.shape[-1]
+    T = int(n_rows if n_rows is not None else (len(rows) if rows is not None else x.shape[0]))
+    xb, (wb, wdt) = _f(x), weight_buffer(w, dtype)
+    yb = _f(y0) if y0 is not None else DeviceBuffer.zeros(max(T, 1) * N * 4)
+    ob = _i(offsets) if offsets is not None else None
+    rb = _i(rows) if rows is not None else None
+    d = DenseDesc(yb.ptr, N, xb.ptr, x.shape[1], wb.ptr, N * K if stacked else 0, wdt, ob.ptr if ob else None, w.shape[0] if stacked else 1,
+                  rb.ptr if rb else None, row_div, T, N, K, int(y0 is not None))
+    check(L.ntk_dense(C.byref(d), None), "ntk_dense")
+    return yb.numpy(np.float32, T * N).reshape(T, N)
+
+
+def rmsnorm_offset(x: np.ndarray, w1: np.ndarray, w2: Optional[np.ndarray], eps: float, offset: float):
+    L = _bind()
+    T, n = x.shape
+    xb, w1b = _f(x), _f(w1)
+    y1 = DeviceBuffer.zeros(T * n * 4)
+    y2 = DeviceBuffer.zeros(T * n * 4) if w2 is not None else None
+    w2b = _f(w2) if w2 is not None else None
+    check(L.ntk_rmsnorm_offset(y1.ptr, w1b.ptr, y2.ptr if y2 else None, w2b.ptr if w2b else None, n, xb.ptr, n, T, n, eps, offset, None), "ntk_rmsnorm_offset")
+    a = y1.numpy(np.float32, T * n).reshape(T, n)
+    return (a, y2.numpy(np.float32, T * n).reshape(T, n)) if y2 else a
+
+
+def latent_prepare(kv: np.ndarray, norm_w: np.ndarray, eps: float, kv_rank: int, rot_dim: int, q: Optional[np.ndarray], heads: int, freq: np.ndarray, mag: float,
+                   dims: int, pos0: int, cache: Optional[np.ndarray] = None, cache_rows: Optional[int] = None):
+    """-> (cache [rows, kv_rank + rot_dim] with rows pos0.. filled, q rotated)"""
+    L = _bind()
+    T, row = kv.shape[0], kv_rank + rot_dim
+    n = cache_rows or (pos0 + T)
+    cb = _f(cache) if cache is not None else DeviceBuffer.zeros(n * row * 4)
+    kb, nb, fb = _f(kv), _f(norm_w), DeviceBuffer.from_numpy(np.ascontiguousarray(freq, np.float64))
+    qb = _f(q) if q is not None else None
+    qd = q.shape[1] // heads if q is not None else rot_dim
+    rot = Rotary(fb.ptr, mag, dims)
+    check(L.ntk_latent_prepare(cb.ptr, row, kb.ptr, kv.shape[1], nb.ptr, eps, kv_rank, rot_dim, qb.ptr if qb else None, q.shape[1] if q is not None else 0, heads, qd,
+                               C.byref(rot), pos0, T, None), "ntk_latent_prepare")
+    return cb.numpy(np.float32, n * row).reshape(n, row), (qb.numpy(np.float32, q.size).reshape(q.shape) if qb else None)
+
+
+def latent_attention(q: np.ndarray, cache: np.ndarray, kv_rank: int, rot_dim: int, heads: int, pos0: int, window: int, scale: float,
+                     K: Optional[np.ndarray] = None, V: Optional[np.ndarray] = None, key0: int = 0) -> np.ndarray:
+    """expanded form when K [nkeys, H * dn] and V [nkeys, H * dv] are given (q [T, H * (dn + dr)]), else the shared form (q [T, H * (R + dr)])"""
+    L = _bind()
+    T, row = q.shape[0], kv_rank + rot_dim
+    qb, cb = _f(q), _f(cache)
+    if K is not None:
+        dn, dv = K.shape[1] // heads, V.shape[1] // heads
+        kb, vb = _f(K), _f(V)
+        out = DeviceBuffer.zeros(T * heads * dv * 4)
+        check(L.ntk_latent_attention(out.ptr, heads * dv, qb.ptr, q.shape[1], kb.ptr, K.shape[1], vb.ptr, V.shape[1], cb.ptr, row, kv_rank, rot_dim, heads, dn, dv, 0,
+                                     pos0, T, key0, window, scale, None, None), "ntk_latent_attention")
+        return out.numpy(np.float32, T * heads * dv).reshape(T, heads * dv)
+    nkeys = pos0 + T
+    sc = DeviceBuffer.zeros(max(int(L.ntk_latent_attention_scratch(T, heads, kv_rank, nkeys)), 1) * 4)
+    out = DeviceBuffer.zeros(T * heads * kv_rank * 4)
+    check(L.ntk_latent_attention(out.ptr, heads * kv_rank, qb.ptr, q.shape[1], None, 0, None, 0, cb.ptr, row, kv_rank, rot_dim, heads, 0, 0, 1, pos0, T, 0, window,
+                                 scale, sc.ptr, None), "ntk_latent_attention")
+    return out.numpy(np.float32, T * heads * kv_rank).reshape(T, heads * kv_rank)
+
+
+def latent_fold_query(q: np.ndarray, w_uk: np.ndarray, heads: int, dn: int, dr: int, dtype: str = "float32") -> np.ndarray:
+    L = _bind()
+    T, R = q.shape[0], w_uk.shape[1]
+    qb, (wb, wdt) = _f(q), weight_buffer(w_uk, dtype)
+    out = DeviceBuffer.zeros(T * heads * (R + dr) * 4)
+    check(L.ntk_latent_fold_query(out.ptr, qb.ptr, q.shape[1], wb.ptr, wdt, T, heads, dn, dr, R, None), "ntk_latent_fold_query")
+    return out.numpy(np.float32, T * heads * (R + dr)).reshape(T, heads * (R + dr))
+
+
+def latent_unfold_value(lat: np.ndarray, w_uv: np.ndarray, heads: int, gate: Optional[np.ndarray] = None, dtype: str = "float32") -> np.ndarray:
+    L = _bind()
+    T, R = lat.shape[0], w_uv.shape[1]
+    dv = w_uv.shape[0] // heads
+    lb, (wb, wdt) = _f(lat), weight_buffer(w_uv, dtype)
+    gb = _f(gate) if gate is not None else None
+    out = DeviceBuffer.zeros(T * heads * dv * 4)
+    check(L.ntk_latent_unfold_value(out.ptr, heads * dv, lb.ptr, wb.ptr, wdt, gb.ptr if gb else None, heads * dv, T, heads, dv, R, None), "ntk_latent_unfold_value")
+    return out.numpy(np.float32, T * heads * dv).reshape(T, heads * dv)
+
+
+def moe_route(h: np.ndarray, w_router: np.ndarray, top: int, shared_gate_w: Optional[np.ndarray] = None):
+    L = _bind()
+    T, n = h.shape
+    E = w_router.shape[0]
+    hb, wb = _f(h), _f(w_router)
+    sb = _f(shared_gate_w) if shared_gate_w is not None else None
+    ids, wts, sg = DeviceBuffer.zeros(T * top * 4), DeviceBuffer.zeros(T * top * 4), DeviceBuffer.zeros(T * 4)
+    check(L.ntk_moe_route(ids.ptr, wts.ptr, sg.ptr if sb else None, hb.ptr, n, wb.ptr, sb.ptr if sb else None, T, n, E, top, None), "ntk_moe_route")
+    return ids.numpy(np.int32, T * top).reshape(T, top), wts.numpy(np.float32, T * top).reshape(T, top), (sg.numpy(np.float32, T) if sb else None)
+
+
+def moe_group(ids: np.ndarray, E: int):
+    L = _bind()
+    T, top = ids.shape
+    ib = _i(ids)
+    off, order, where = DeviceBuffer.zeros((E + 1) * 4), DeviceBuffer.zeros(T * top * 4), DeviceBuffer.zeros(T * top * 4)
+    check(L.ntk_moe_group(off.ptr, order.ptr, where.ptr, ib.ptr, T, top, E, None), "ntk_moe_group")
+    return off.numpy(np.int32, E + 1), order.numpy(np.int32, T * top), where.numpy(np.int32, T * top)
+
+
+def clipped_glu(gu: np.ndarray, limit: float, alpha: float = 1.702) -> np.ndarray:
+    L = _bind()
+    rows, ff = gu.shape[0], gu.shape[1] // 2
+    gb = _f(gu)
+    out = DeviceBuffer.zeros(rows * ff * 4)
+    check(L.ntk_clipped_glu(out.ptr, gb.ptr, rows, ff, limit, alpha, None), "ntk_clipped_glu")
+    return out.numpy(np.float32, rows * ff).reshape(rows, ff)
+
+
+def moe_combine(x, mix, d, where, wts, shared=None, sgate=None) -> np.ndarray:
+    L = _bind()
+    T, n = x.shape
+    top = wts.shape[1]
+    xb, db, wb, tb = _f(x), _f(d), _i(where), _f(wts)
+    mb = _f(mix) if mix is not None else None
+    sb = _f(shared) if shared is not None else None
+    gb = _f(sgate) if sgate is not None else None
+    check(L.ntk_moe_combine(xb.ptr, mb.ptr if mb else None, db.ptr, wb.ptr, tb.ptr, sb.ptr if sb else None, gb.ptr if gb else None, T, top, n, None), "ntk_moe_combine")
+    return xb.numpy(np.float32, T * n).reshape(T, n)

@@ -32,10 +32,6 @@ def norm_plain(x, w, eps):
     return rms_unit(x, eps) * w
 
 
-def gelu_tanh(z):
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
-
-
 def rotary_frequencies(rot):
     """Per pair i: the angle step per position and the factor on cos and sin (1 without scaling)."""
     dims, base = int(rot["dims"]), float(rot["base"])
@@ -69,14 +65,23 @@ def rotate_pairs(x, pos, rot):
     return out
 
 
-def visible(T, window):
-    """[T, T] bool: query i sees key j.  window None: every j <= i; else the last `window` positions, itself included."""
-    i = torch.arange(T)[:, None]
-    j = torch.arange(T)[None, :]
+def visible(qpos, kpos, window):
+    """[Tq, Tk] bool: the query at position i sees the key at position j.  window None: every j <= i; else the last `window` positions, itself
+    included."""
+    i = torch.as_tensor(qpos)[:, None]
+    j = torch.as_tensor(kpos)[None, :]
     m = j <= i
     if window is not None:
-        m &= (i - j) < window
+        m = m & ((i - j) < window)
     return m
+
+
+def attend(qn, qr, kn, kr, v, qpos, kpos, window, scale):
+    """Softmax attention with a two-part score.  qn [Tq, H, dn], qr [Tq, H, dr] (rotated), kn [Tk, H, dn], kr [Tk, dr] (rotated, one for all heads),
+    v [Tk, H, dv] -> [Tq, H, dv]."""
+    s = (torch.einsum("thd,shd->hts", qn, kn) + torch.einsum("thd,sd->hts", qr, kr)) * scale
+    s = s.masked_fill(~visible(qpos, kpos, window)[None], float("-inf"))
+    return torch.einsum("hts,shd->thd", torch.softmax(s, dim=-1), v)
 
 
 def latent_attention(h, w, pre, mx, eps, pos=None):
@@ -93,15 +98,11 @@ def latent_attention(h, w, pre, mx, eps, pos=None):
     kv = h @ w[pre + "dkv"].T
     c = norm_plain(kv[:, :R], w[pre + "dkv.norm"], eps)     # [T, R]
     kr = rotate_pairs(kv[:, R:], pos, mx["rot"])            # [T, dr], one for all heads
-    qr = rotate_pairs(q[:, :, dn:].transpose(0, 1), pos, mx["rot"])   # [H, T, dr]
+    qr = rotate_pairs(q[:, :, dn:].transpose(0, 1), pos, mx["rot"]).transpose(0, 1)   # [T, H, dr]
     kn = (c @ w[pre + "uk"].T).view(T, H, dn)
     v = (c @ w[pre + "uv"].T).view(T, H, dv)
-    s = torch.einsum("thd,shd->hts", q[:, :, :dn], kn) + torch.einsum("htd,sd->hts", qr, kr)
-    s = s * float(mx["scale"])
     window = int(mx["mask"]["size"]) if mx.get("mask") else None
-    s = s.masked_fill(~visible(T, window)[None], float("-inf"))
-    p = torch.softmax(s, dim=-1)
-    o = torch.einsum("hts,shd->thd", p, v).reshape(T, H * dv)
+    o = attend(q[:, :, :dn], qr, kn, kr, v, pos, pos, window, float(mx["scale"])).reshape(T, H * dv)
     o = o * torch.sigmoid(h @ w[pre + "g"].T)
     return o @ w[pre + "o"].T
 
@@ -273,13 +274,22 @@ def load_model(folder):
     return cfg, w
 
 
+def greedy(cfg, w, prompt, n):
+    """n tokens chosen by the largest logit, each from a whole forward of everything so far."""
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(torch.argmax(forward(cfg, w, toks)[-1])))
+    return toks[len(prompt):]
+
+
 def small_config(layers=("latent_attention", "latent_attention_2"), width=64, vocab=96, heads=2, dim=16, rot_dim=8, vdim=24, kv_rank=32,
-                 q_rank=24, window=5, experts=4, top=2, ff=32, shared_ff=48, loop=None, scaling=True, limit=1.5, eps=1e-5, base=10000.0):
+                 q_rank=24, window=5, experts=4, top=2, ff=32, shared_ff=48, loop=None, scaling=True, limit=1.5, eps=1e-5, base=10000.0,
+                 rot_dims=None, mlp_on=None):
     """A configuration whose sizes all differ from each other, so that a swapped pair shows."""
     ls = []
     for k, t in enumerate(layers):
         mx = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "scale": 1.0 / math.sqrt(dim + rot_dim),
-              "rot": {"base": base * (1 + k), "dims": rot_dim}}
+              "rot": {"base": base * (1 + k), "dims": rot_dims or rot_dim}}
         if t == "latent_attention":
             mx["q_rank"] = q_rank
             if scaling:
@@ -289,7 +299,7 @@ def small_config(layers=("latent_attention", "latent_attention_2"), width=64, vo
         ml = {"kind": "moe", "expert": {"ff": ff, "limit": limit}, "router": {"experts": experts, "top": top}}
         if shared_ff:
             ml["shared"] = {"ff": shared_ff, "limit": limit * 0.75}
-        ls.append({"type": t, "mixer": mx, "mlp": ml})
+        ls.append({"type": t, "mixer": mx, "mlp": ml if (mlp_on is None or mlp_on[k]) else None})
     cfg = {"architecture": "Fabolorn", "layers": ls, "norm": {"eps": eps}, "vocab": vocab, "width": width}
     if loop:
         cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}

@@ -25,7 +25,7 @@ def declared_functions(header, where="include"):
     return sorted(set(re.findall(r"\b((?:ntk|nt)_[a-z0-9_]+)\s*\(", src)) - {"nt_engine_t", "nt_tokenizer_t"})
 
 
-@pytest.mark.parametrize("header", ["ntk.h", "ntk_engine.h", "ntransformer.h"])
+@pytest.mark.parametrize("header", ["ntk.h", "ntk_engine.h", "ntk_layers.h", "ntransformer.h"])
 def test_library_exports_every_declared_symbol(header):
     L = _lib.lib()
     names = declared_functions(header)
@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol(header):
 
 
 def test_library_exports_nothing_but_the_headers():
-    """-fvisibility=hidden: the dynamic symbol table of the shipping library holds the C functions the three headers declare and nothing else of ours
+    """-fvisibility=hidden: the dynamic symbol table of the shipping library holds the C functions the four headers declare and nothing else of ours
     (hipcc's kernel stubs / __hip_* registration symbols aside)."""
     import shutil
     import subprocess
@@ -44,7 +44,7 @@ def test_library_exports_nothing_but_the_headers():
     out = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], capture_output=True, text=True).stdout
     have = {l.split()[-1] for l in out.splitlines() if " T " in l}
     ours = {n for n in have if n.startswith(("ntk_", "nt_"))}
-    declared = set(declared_functions("ntk.h")) | set(declared_functions("ntk_engine.h")) | set(declared_functions("ntransformer.h"))
+    declared = set(declared_functions("ntk.h")) | set(declared_functions("ntk_engine.h")) | set(declared_functions("ntk_layers.h")) | set(declared_functions("ntransformer.h"))
     assert not (ours - declared), sorted(ours - declared)
 
 
