@@ -60,6 +60,12 @@ def parse():
     ap.add_argument("--cpu-tokens", type=int, default=128, help="-n of the reference CLI run that is the CPU baseline (BASELINE config 1: 128)")
     ap.add_argument("--no-also", action="store_true", help="skip the other BASELINE configurations (8B Q4_K_M, 70B Q4_K_M, 70B Q6_K, 8B Q8_0 behind 3900- and 32768-token prompts)")
     ap.add_argument("--no-pmc-note", action="store_true")
+    ap.add_argument("--family", default="", choices=["", "fabolorn"],
+                    help="instead of the default workload: prompt and decode throughput of a layer-list family on synthetic real-sized layers, beside the "
+                         "Llama path at equal width / heads / active feed-forward width (F16 and Q8_0); one JSON line of its own")
+    ap.add_argument("--family-size", default="lite", choices=["tiny", "lite", "mid"])
+    ap.add_argument("--family-layers", type=int, default=2)
+    ap.add_argument("--family-dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prompt-bench", type=int, default=1024, help="also time one prompt pass of this many tokens (0 = skip); reported under config.prompt_pass")
     return ap.parse_args()
 
@@ -382,8 +388,78 @@ def roofline_block(args, model, mix, r):
             "token_ms_by_class_eager": {"gemv": round(r["ms"][0], 4), "attention": round(r["ms"][1], 4), "other": round(r["ms"][2], 4)}}
 
 
+def run_family(args):
+    """--family fabolorn: a synthetic model folder of `--family-layers` real-sized layers (ntransformer_amd/synth_folder.py), a prompt pass of
+    --prompt-bench tokens (second of two runs) and --steps decoded tokens behind it through the slot cache; then the Llama path with the same width,
+    heads (head size 128), layers, vocabulary and ACTIVE feed-forward width (top x ff + shared ff) as F16 and as Q8_0, same prompt and decode."""
+    import shutil
+    import tempfile
+    import numpy as np
+    from ntransformer_amd import _lib, synth_folder
+    from ntransformer_amd import engine as E
+    L = _lib.lib()
+    _lib.check(L.ntk_device_init(0), "ntk_device_init")
+    cfg = synth_folder.fabolorn_config(args.family_size, args.family_layers)
+    p = synth_folder.PRESETS[args.family_size]
+    T, ctx = args.prompt_bench or 1024, max(args.ctx, (args.prompt_bench or 1024) + args.steps + args.warmup + 8)
+    tmp = tempfile.mkdtemp(prefix="ntk_family_")
+    rng = np.random.Generator(np.random.Philox(key=[20260925, 7]))
+    prompt = [int(t) for t in rng.integers(0, p["vocab"], T)]
+    out = {}
+    try:
+        nbytes = synth_folder.write_folder(tmp, cfg)
+        eng = E.Engine()
+        eng.load_folder(tmp, max_context=ctx, dtype=args.family_dtype)
+        s = eng.seq_acquire()
+        eng.seq_forward(s, prompt, want=[T - 1])
+        eng.seq_release(s)
+        s = eng.seq_acquire()
+        t0 = time.perf_counter()
+        lg = eng.seq_forward(s, prompt, want=[T - 1])
+        t_prompt = time.perf_counter() - t0
+        tok = int(lg[0].argmax())
+        for _ in range(args.warmup):
+            tok = int(eng.seq_forward(s, [tok], want=[0])[0].argmax())
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            tok = int(eng.seq_forward(s, [tok], want=[0])[0].argmax())
+        t_dec = time.perf_counter() - t0
+        out["fabolorn"] = {"prompt_tok_s": round(T / t_prompt, 1), "decode_tok_s": round(args.steps / t_dec, 1), "decode_ms_per_token": round(1e3 * t_dec / args.steps, 3),
+                           "weight_bytes": eng.weight_bytes(), "file_bytes": nbytes}
+        eng.close()
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    for mix in ("F16", "Q8_0"):
+        try:
+            inter = p["top"] * p["ff"] + p["shared_ff"]
+            inter -= inter % 256
+            spec = E.SynthSpec(p["width"], inter, args.family_layers, p["width"] // 128, p["width"] // 128, p["vocab"], ctx, 1e-5, 500000.0, 1, 2, mix.encode(), 20260925)
+            eng = E.Engine()
+            eng.load_synthetic(spec, ctx)
+            eng.forward(prompt, 0)
+            t0 = time.perf_counter()
+            eng.forward(prompt, 0)
+            t_prompt = time.perf_counter() - t0
+            first = eng.generate_tokens(prompt, 1, temperature=0.0, repeat_penalty=1.0, stop_at_eos=False)
+            warm = eng.decode_greedy_steps(first[0], T, args.warmup) if args.warmup else first
+            t0 = time.perf_counter()
+            eng.decode_greedy_steps(warm[-1], T + args.warmup, args.steps)
+            t_dec = time.perf_counter() - t0
+            out["llama_" + mix.lower()] = {"prompt_tok_s": round(T / t_prompt, 1), "decode_tok_s": round(args.steps / t_dec, 1),
+                                           "decode_ms_per_token": round(1e3 * t_dec / args.steps, 3), "weight_bytes": eng.weight_bytes(), "inter": inter}
+            eng.close()
+        except Exception as e:
+            out["llama_" + mix.lower()] = {"error": repr(e)}
+    print(json.dumps({"metric": "fabolorn_decode_tokens_per_s", "value": out["fabolorn"]["decode_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+                      "warmup": args.warmup, "ms_per_step": out["fabolorn"]["decode_ms_per_token"], "higher_is_better": True, "dtype": args.family_dtype,
+                      "data": "synthetic", "config": {"family": "fabolorn", "size": args.family_size, "layers": args.family_layers, "prompt_tokens": T,
+                                                      "preset": p}, "results": out}))
+
+
 def main():
     args = parse()
+    if args.family:
+        return run_family(args)
     rank = int(os.environ.get("RANK", "0"))
     local_rank = int(os.environ.get("LOCAL_RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))

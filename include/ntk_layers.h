@@ -34,7 +34,11 @@ typedef struct ntk_dense_desc {
     const int* rows; int row_div;
     int T, N, K;
     int accumulate;
+    /* glu_ff > 0 (only with T <= ntk_dense_few_rows(), N == 2 * glu_ff, no accumulate): W holds glu_ff gate rows then glu_ff up rows and
+     * Y[r][f] = g' * sigmoid(glu_alpha * g') * (u' + 1), g' = min(gate, glu_limit), u' = clamp(up, -glu_limit, glu_limit) -- the product and ntk_clipped_glu in one launch */
+    int glu_ff; float glu_limit, glu_alpha;
 } ntk_dense_desc;
+int ntk_dense_few_rows(void);   /* up to this many rows a product takes the row-streaming form */
 int ntk_dense(const ntk_dense_desc* d, void* stream);
 /* the plain case: Y[T][N] = X[T][K] . W[N][K]^T */
 int ntk_dense_linear(float* Y, int ldy, const float* X, int ldx, const void* W, int wdtype, int T, int N, int K, int accumulate, void* stream);

@@ -13,6 +13,7 @@ namespace nt {
         if (st__ != NTK_OK) return st__;      \
     } while (0)
 
+static constexpr float kGluAlpha = 1.702f;   // the design fixes the slope of the experts' gate activation
 static FamilyRegistrar reg_fabolorn("Fabolorn", [] { return std::unique_ptr<SequenceModel>(new LayerStackModel()); });
 
 LayerStackModel::~LayerStackModel() {
@@ -299,7 +300,7 @@ int LayerStackModel::alloc_buffers() {
               fl(&att_, C * max_hdv_) && fl(&kx_, ctx * max_hdn_) && fl(&vx_, ctx * max_hdv_) && fl(&mix_, C * W) && fl(&xw_, C * W) && fl(&hn_, C * W) &&
               in(&tokens_dev_, C) && in(&want_dev_, C);
     size_t sc = 0;
-    for (const auto& L : layers_) sc = std::max(sc, (size_t)kSharedRows * L.mix.heads * 32 * (2 + (size_t)L.mix.kv_rank));
+    for (const auto& L : layers_) sc = std::max(sc, ntk_latent_attention_scratch(kSharedRows, L.mix.heads, L.mix.kv_rank, opt_.max_context));
     ok = ok && fl(&scratch_, sc);
     if (max_top_ > 0) {
         const size_t P = C * max_top_;
@@ -363,8 +364,14 @@ int LayerStackModel::run_experts(const ClippedExperts& ex, const float* h, float
     ntk_dense_desc d{};
     d.Y = gu; d.ldy = 2 * ex.ff; d.X = h; d.ldx = W; d.W = ex.gate_up.ptr; d.wstride = ex.gate_up.stride(); d.wdtype = ex.gate_up.dtype;
     d.offsets = offsets; d.G = ex.gate_up.count; d.rows = order; d.row_div = top; d.T = rows; d.N = 2 * ex.ff; d.K = W; d.accumulate = 0;
-    LS_TRY(ntk_dense(&d, stream_));
-    LS_TRY(ntk_clipped_glu(act, gu, rows, ex.ff, ex.limit, 1.702f, stream_));
+    if (rows <= ntk_dense_few_rows()) {   // decoding: the activation inside the product's launch
+        d.Y = act; d.ldy = ex.ff; d.glu_ff = ex.ff; d.glu_limit = ex.limit; d.glu_alpha = kGluAlpha;
+        LS_TRY(ntk_dense(&d, stream_));
+        d.glu_ff = 0;
+    } else {
+        LS_TRY(ntk_dense(&d, stream_));
+        LS_TRY(ntk_clipped_glu(act, gu, rows, ex.ff, ex.limit, kGluAlpha, stream_));
+    }
     d.Y = out; d.ldy = W; d.X = act; d.ldx = ex.ff; d.W = ex.down.ptr; d.wstride = ex.down.stride(); d.wdtype = ex.down.dtype;
     d.rows = nullptr; d.row_div = 1; d.N = W; d.K = ex.ff;
     return ntk_dense(&d, stream_);

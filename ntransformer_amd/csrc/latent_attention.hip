@@ -196,85 +196,226 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(const AttnArgs a)
     }
 }
 
-// merge of the partial states of one (token, head): grid (rows), state index = row as the attention kernel numbered it
-__global__ __launch_bounds__(64) void latent_attention_merge_kernel(float* out, int ldo, const float* scratch, int splits, int nV, int H) {
-    const int r = blockIdx.x;   // shared numbering: r = t * H + h
+// ------------------------------------------------------------------------------------------------------------------- the shared form (decoding)
+// Keys and values are the cache rows themselves, so a workgroup loads a tile of KB = 32 rows [latent | rotated] ONCE (all requests in flight together) and
+// uses it for every (token, head) row of its tile of 16: thread (key, row pair) forms two scores over the whole row, sixteen threads run the online softmax
+// of their row, then thread r sums the weighted latents column r of all 16 rows.  The tiles of 32 keys go round `splits` workgroups; each leaves one
+// (max, sum, vector) state per row and latent_attention_merge_kernel adds them.
+constexpr int KB = 32, SROWS = 16;
+struct SharedArgs {
+    const float* q; int ldq;          // [T][H][R + dr], ldq floats between tokens
+    const float* cache; int row;      // cache rows
+    int R, dr, H, pos0, T, window, splits;
+    float scale;
+    float* scratch;                   // [rows][splits][2 + R]
+};
+
+__global__ __launch_bounds__(256) void latent_attention_shared_kernel(const SharedArgs a) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int DK = a.R + a.dr;
+    const int DKP = ((DK + 3) & ~3) + 4;           // rows 16-byte aligned, 4 banks apart
+    float* Ks = lds;                               // [KB][DKP]
+    float* Qs = Ks + KB * DKP;                     // [SROWS][DKP]
+    float* Ps = Qs + SROWS * DKP;                  // [SROWS][KB]
+    float* ms = Ps + SROWS * KB;                   // [SROWS] running max
+    float* ls = ms + SROWS;                        // [SROWS] running sum
+    float* cr = ls + SROWS;                        // [SROWS] correction of this tile
+    const int tid = threadIdx.x;
+    const int n_rows = a.T * a.H, row0 = blockIdx.x * SROWS;
+    const int last_row = min(row0 + SROWS, n_rows) - 1;
+    const int pmin = a.pos0 + row0 / a.H, pmax = a.pos0 + last_row / a.H;
+    const int jlo = a.window > 0 ? max(0, pmin - a.window + 1) : 0, jhi = pmax;
+    for (int idx = tid; idx < SROWS * DKP; idx += 256) {
+        const int i = idx / DKP, d = idx % DKP, r = row0 + i;
+        Qs[idx] = (r < n_rows && d < DK) ? a.q[(long long)(r / a.H) * a.ldq + (long long)(r % a.H) * DK + d] : 0.0f;
+    }
+    if (tid < SROWS) { ms[tid] = -INFINITY; ls[tid] = 0.0f; }
+    const int key = tid % KB, rg = tid / KB;       // scores: rows 2 rg, 2 rg + 1
+    const int rpos0 = row0 + 2 * rg < n_rows ? a.pos0 + (row0 + 2 * rg) / a.H : -1;
+    const int rpos1 = row0 + 2 * rg + 1 < n_rows ? a.pos0 + (row0 + 2 * rg + 1) / a.H : -1;
+    constexpr int RC = 2;                          // latent columns per thread: R <= 512
+    float acc[RC][SROWS];
+#pragma unroll
+    for (int c = 0; c < RC; ++c)
+#pragma unroll
+        for (int i = 0; i < SROWS; ++i) acc[c][i] = 0.0f;
+    const bool vec4 = (DK % 4 == 0) && (a.row % 4 == 0) && !((uintptr_t)a.cache & 15);
+    int tile = 0;
+    for (int j0 = jlo; j0 <= jhi; j0 += KB, ++tile) {
+        if (tile % a.splits != (int)blockIdx.y) continue;
+        const int nk = min(KB, jhi + 1 - j0);
+        __syncthreads();                           // the previous tile is used up (and Qs / ms are written)
+        if (vec4) {
+            const int q4 = DK / 4;
+            for (int idx = tid; idx < KB * q4; idx += 256) {
+                const int k = idx / q4, c4 = idx % q4;
+                float4 v = float4{0.f, 0.f, 0.f, 0.f};
+                if (k < nk) v = *reinterpret_cast<const float4*>(a.cache + (long long)(j0 + k) * a.row + 4 * c4);
+                *reinterpret_cast<float4*>(Ks + k * DKP + 4 * c4) = v;
+            }
+        } else {
+            for (int idx = tid; idx < KB * DKP; idx += 256) {
+                const int k = idx / DKP, d = idx % DKP;
+                Ks[idx] = (k < nk && d < DK) ? a.cache[(long long)(j0 + k) * a.row + d] : 0.0f;
+            }
+        }
+        __syncthreads();
+        // ---- scores
+        float s0 = 0.0f, s1 = 0.0f;
+        const float* kr = Ks + key * DKP;
+        const float* qa = Qs + (2 * rg) * DKP;
+        const float* qb = qa + DKP;
+        for (int d = 0; d < DK; d += 4) {          // (entries past DK are zero on both sides)
+            const float4 kv = *reinterpret_cast<const float4*>(kr + d), xa = *reinterpret_cast<const float4*>(qa + d), xb = *reinterpret_cast<const float4*>(qb + d);
+            s0 = fmaf(xa.x, kv.x, s0); s0 = fmaf(xa.y, kv.y, s0); s0 = fmaf(xa.z, kv.z, s0); s0 = fmaf(xa.w, kv.w, s0);
+            s1 = fmaf(xb.x, kv.x, s1); s1 = fmaf(xb.y, kv.y, s1); s1 = fmaf(xb.z, kv.z, s1); s1 = fmaf(xb.w, kv.w, s1);
+        }
+        const int j = j0 + key;
+        const bool v0 = key < nk && rpos0 >= 0 && j <= rpos0 && (a.window <= 0 || rpos0 - j < a.window);
+        const bool v1 = key < nk && rpos1 >= 0 && j <= rpos1 && (a.window <= 0 || rpos1 - j < a.window);
+        Ps[(2 * rg) * KB + key] = v0 ? s0 * a.scale : -INFINITY;
+        Ps[(2 * rg + 1) * KB + key] = v1 ? s1 * a.scale : -INFINITY;
+        __syncthreads();
+        // ---- online softmax, one thread per row
+        if (tid < SROWS) {
+            float* p = Ps + tid * KB;
+            float mc = -INFINITY;
+            for (int k = 0; k < KB; ++k) mc = fmaxf(mc, p[k]);
+            const float mn = fmaxf(ms[tid], mc), msafe = mn == -INFINITY ? 0.0f : mn;
+            const float corr = ms[tid] == -INFINITY ? 0.0f : expf(ms[tid] - msafe);
+            float sum = 0.0f;
+            for (int k = 0; k < KB; ++k) { const float e = p[k] == -INFINITY ? 0.0f : expf(p[k] - msafe); p[k] = e; sum += e; }
+            ls[tid] = ls[tid] * corr + sum;
+            ms[tid] = mn;
+            cr[tid] = corr;
+        }
+        __syncthreads();
+        // ---- weighted latents: thread -> column tid (+ 256)
+#pragma unroll
+        for (int c = 0; c < RC; ++c) {
+            const int r = tid + 256 * c;
+            if (r < a.R) {
+#pragma unroll
+                for (int i = 0; i < SROWS; ++i) acc[c][i] *= cr[i];
+                for (int k = 0; k < KB; k += 4) {
+                    const float x0 = Ks[(k + 0) * DKP + r], x1 = Ks[(k + 1) * DKP + r], x2 = Ks[(k + 2) * DKP + r], x3 = Ks[(k + 3) * DKP + r];
+#pragma unroll
+                    for (int i = 0; i < SROWS; ++i) {
+                        const float4 p4 = *reinterpret_cast<const float4*>(Ps + i * KB + k);
+                        acc[c][i] = fmaf(p4.x, x0, acc[c][i]); acc[c][i] = fmaf(p4.y, x1, acc[c][i]);
+                        acc[c][i] = fmaf(p4.z, x2, acc[c][i]); acc[c][i] = fmaf(p4.w, x3, acc[c][i]);
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+    for (int i = 0; i < SROWS; ++i) {
+        if (row0 + i >= n_rows) break;
+        float* st = a.scratch + ((long long)(row0 + i) * a.splits + blockIdx.y) * (2 + a.R);
+        if (tid == 0) { st[0] = ms[i]; st[1] = ls[i]; }
+#pragma unroll
+        for (int c = 0; c < RC; ++c)
+            if (tid + 256 * c < a.R) st[2 + tid + 256 * c] = acc[c][i];
+    }
+}
+
+// merge of the partial states of one (token, head) row: weights of the states first, then every thread sums its columns over the states
+__global__ __launch_bounds__(256) void latent_attention_merge_kernel(float* out, int ldo, const float* scratch, int splits, int nV, int H) {
+    __shared__ float wt[256];
+    __shared__ float red[16];
+    const int r = blockIdx.x;   // r = t * H + h
     const float* st = scratch + (long long)r * splits * (2 + nV);
     float mx = -INFINITY;
-    for (int s = 0; s < splits; ++s) mx = fmaxf(mx, st[(long long)s * (2 + nV)]);
+    for (int s = threadIdx.x; s < splits; s += 256) mx = fmaxf(mx, st[(long long)s * (2 + nV)]);
+    mx = block_max(mx, red);
     float den = 0.0f;
-    for (int s = 0; s < splits; ++s) {
-        const float ms = st[(long long)s * (2 + nV)];
-        if (ms != -INFINITY) den += st[(long long)s * (2 + nV) + 1] * expf(ms - mx);
+    for (int s = threadIdx.x; s < splits; s += 256) {
+        const float m = st[(long long)s * (2 + nV)];
+        const float w = m == -INFINITY ? 0.0f : expf(m - mx);
+        wt[s] = w;
+        den += w * st[(long long)s * (2 + nV) + 1];
     }
+    den = block_sum(den, red);   // (its barriers publish wt)
     const float inv = den > 0.0f ? 1.0f / den : 0.0f;
     float* o = out + (long long)(r / H) * ldo + (long long)(r % H) * nV;
-    for (int v = threadIdx.x; v < nV; v += 64) {
+    for (int v = threadIdx.x; v < nV; v += 256) {
         float s2 = 0.0f;
-        for (int s = 0; s < splits; ++s) {
-            const float ms = st[(long long)s * (2 + nV)];
-            if (ms != -INFINITY) s2 = fmaf(st[(long long)s * (2 + nV) + 2 + v], expf(ms - mx), s2);
-        }
+        for (int s = 0; s < splits; ++s) s2 = fmaf(st[(long long)s * (2 + nV) + 2 + v], wt[s], s2);
         o[v] = s2 * inv;
     }
 }
 
 // ------------------------------------------------------------------------------------------------------------------- fold / unfold
-// qf[t][h][r] = sum_d q[t][h][d] W_uk[h * dn + d][r]; rotated part copied behind.  grid (H, T)
+// qf[t][h][r] = sum_d q[t][h][d] W_uk[h * dn + d][r]; rotated part copied behind.  grid (R / 64, H, T): 64 columns per workgroup, the d range in
+// four parts (one per wave), added through LDS in wave order
 template <typename WT>
 __global__ __launch_bounds__(256) void latent_fold_query_kernel(float* qf, const float* q, int ldq, const WT* w, int H, int dn, int dr, int R) {
-    extern __shared__ float qs[];
-    const int h = blockIdx.x, t = blockIdx.y;
+    extern __shared__ float qs[];      // [dn + dr] then [4][64] partial sums
+    float* part = qs + dn + dr;
+    const int h = blockIdx.y, t = blockIdx.z;
     const float* qh = q + (long long)t * ldq + (long long)h * (dn + dr);
     float* o = qf + ((long long)t * H + h) * (R + dr);
     for (int d = threadIdx.x; d < dn + dr; d += 256) qs[d] = qh[d];
     __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = blockIdx.x * 64 + lane;
+    const int per = (dn + 3) / 4, d0 = wave * per, d1 = min(d0 + per, dn);
     const WT* wh = w + (long long)h * dn * R;
-    for (int r = threadIdx.x; r < R; r += 256) {
-        float s = 0.0f;
-        for (int d = 0; d < dn; ++d) {
+    float s = 0.0f;
+    if (r < R) {
+#pragma unroll 8
+        for (int d = d0; d < d1; ++d) {
             float wv;
             if constexpr (sizeof(WT) == 2) wv = __uint_as_float((uint32_t)wh[(long long)d * R + r] << 16); else wv = wh[(long long)d * R + r];
             s = fmaf(qs[d], wv, s);
         }
-        o[r] = s;
     }
-    for (int d = threadIdx.x; d < dr; d += 256) o[R + d] = qs[dn + d];
+    part[wave * 64 + lane] = s;
+    __syncthreads();
+    if (wave == 0 && r < R) o[r] = ((part[lane] + part[64 + lane]) + part[128 + lane]) + part[192 + lane];
+    if (blockIdx.x == 0)
+        for (int d = threadIdx.x; d < dr; d += 256) o[R + d] = qs[dn + d];
 }
 
-// out[t][h * dv + v] = W_uv[h * dv + v][:] . lat[t][h][:] (* sigmoid(gate));  grid (H, T), one wave per output
+// out[t][h * dv + v] = W_uv[h * dv + v][:] . lat[t][h][:] (* sigmoid(gate));  grid (dv / 16, H, T): a wave owns 4 outputs and walks their rows together
 template <typename WT>
 __global__ __launch_bounds__(256) void latent_unfold_value_kernel(float* out, int ldo, const float* lat, const WT* w, const float* gate, int ldg, int H, int dv,
                                                                  int R) {
     extern __shared__ float ls[];
-    const int h = blockIdx.x, t = blockIdx.y;
+    const int h = blockIdx.y, t = blockIdx.z;
     const float* lh = lat + ((long long)t * H + h) * R;
     for (int r = threadIdx.x; r < R; r += 256) ls[r] = lh[r];
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int v = wave; v < dv; v += 4) {
-        const WT* wr = w + ((long long)h * dv + v) * R;
-        float s = 0.0f;
-        for (int r = lane; r < R; r += 64) {
-            float wv;
-            if constexpr (sizeof(WT) == 2) wv = __uint_as_float((uint32_t)wr[r] << 16); else wv = wr[r];
-            s = fmaf(wv, ls[r], s);
+    const int v0 = blockIdx.x * 16 + wave * 4;
+    if (v0 >= dv) return;
+    const WT* wr[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) wr[i] = w + ((long long)h * dv + min(v0 + i, dv - 1)) * R;
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int r = lane; r < R; r += 64) {
+        float wv[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if constexpr (sizeof(WT) == 2) wv[i] = __uint_as_float((uint32_t)wr[i][r] << 16); else wv[i] = wr[i][r];
         }
-        s = wave_sum_lane63(s);
-        if (lane == 63) {
-            if (gate) s *= 1.0f / (1.0f + expf(-gate[(long long)t * ldg + h * dv + v]));
-            out[(long long)t * ldo + h * dv + v] = s;
+        const float x = ls[r];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[i] = fmaf(wv[i], x, s[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float tsum = wave_sum_lane63(s[i]);
+        if (lane == 63 && v0 + i < dv) {
+            if (gate) tsum *= 1.0f / (1.0f + expf(-gate[(long long)t * ldg + h * dv + v0 + i]));
+            out[(long long)t * ldo + h * dv + v0 + i] = tsum;
         }
     }
 }
 
-static int attention_splits(int rows, int nkeys) {
-    const int blocks = (rows + QROWS - 1) / QROWS, chunks = (nkeys + KCH - 1) / KCH;
-    if (blocks >= 128 || chunks < 4) return 1;
-    int s = chunks / 2;
-    if (s > 32) s = 32;
-    while (s > 1 && blocks * s > 1024) --s;
-    return s < 1 ? 1 : s;
+static int shared_splits(int nkeys) {       // workgroups per row tile: one per tile of KB keys, at most 128
+    const int tiles = (nkeys + KB - 1) / KB + 1;     // (+ 1: a tile's first key is the window's, not a multiple of KB)
+    return tiles < 1 ? 1 : tiles > 128 ? 128 : tiles;
 }
 
 }  // namespace ntk
@@ -293,8 +434,7 @@ int ntk_latent_prepare(float* cache, int row, const float* kv, int ldkv, const f
 }
 
 size_t ntk_latent_attention_scratch(int T, int H, int vdim_or_rank, int nkeys) {
-    const int s = attention_splits(T * H, nkeys);
-    return s > 1 ? (size_t)T * H * s * (2 + vdim_or_rank) : 0;
+    return (size_t)T * H * shared_splits(nkeys) * (2 + vdim_or_rank);
 }
 
 int ntk_latent_attention(float* out, int ldo, const float* q, int ldq, const float* K, int ldk, const float* V, int ldv, const float* cache, int row,
@@ -304,56 +444,58 @@ int ntk_latent_attention(float* out, int ldo, const float* q, int ldq, const flo
     if (!shared && (!K || !V)) return NTK_E_NULL;
     if (T < 0 || H <= 0 || kv_rank <= 0 || rot_dim < 0 || pos0 < 0 || key0 < 0 || row < kv_rank + rot_dim) return NTK_E_SHAPE;
     if (T == 0) return NTK_OK;
+    hipStream_t s = resolve_stream(stream);
+    if (shared) {
+        if (!scratch) return NTK_E_NULL;
+        if (kv_rank > 512) return NTK_E_SHAPE;
+        SharedArgs sa{};
+        sa.q = q; sa.ldq = ldq; sa.cache = cache; sa.row = row; sa.R = kv_rank; sa.dr = rot_dim; sa.H = H; sa.pos0 = pos0; sa.T = T; sa.window = window;
+        sa.scale = scale; sa.scratch = scratch;
+        const int nkeys = window > 0 ? (window + T - 1 < pos0 + T ? window + T - 1 : pos0 + T) : pos0 + T;
+        sa.splits = shared_splits(nkeys);
+        const int rows = T * H, DKP = ((kv_rank + rot_dim + 3) & ~3) + 4;
+        const size_t lds = ((size_t)(KB + SROWS) * DKP + SROWS * KB + 3 * SROWS) * sizeof(float);
+        if (lds > 156 * 1024) return NTK_E_SHAPE;
+        static bool raised_s = false;   // (idempotent: a race sets the same attribute twice)
+        if (!raised_s) { NTK_HIP_TRY(hipFuncSetAttribute((const void*)latent_attention_shared_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024)); raised_s = true; }
+        hipLaunchKernelGGL(latent_attention_shared_kernel, dim3((rows + SROWS - 1) / SROWS, sa.splits), dim3(256), lds, s, sa);
+        int st = last_launch_status();
+        if (st != NTK_OK) return st;
+        hipLaunchKernelGGL(latent_attention_merge_kernel, dim3(rows), dim3(256), 0, s, out, ldo, (const float*)scratch, sa.splits, kv_rank, H);
+        return last_launch_status();
+    }
+    if (dn <= 0 || dv <= 0) return NTK_E_SHAPE;
     AttnArgs a{};
     a.out = out; a.ldo = ldo; a.q = q; a.ldq = ldq;
     a.kB = cache + kv_rank; a.ldB = row; a.nB = rot_dim;
-    a.H = H; a.shared = shared; a.pos0 = pos0; a.T = T; a.window = window; a.scale = scale;
-    int rows, nkeys;
-    if (shared) {
-        a.kA = cache; a.ldA = row; a.nA = kv_rank; a.hA = 0;
-        a.v = cache; a.ldV = row; a.nV = kv_rank; a.hV = 0;
-        a.keyA0 = 0;
-        rows = T * H;
-        nkeys = window > 0 ? (window + T < pos0 + T ? window + T : pos0 + T) : pos0 + T;
-        a.splits = attention_splits(rows, nkeys);
-        if (a.splits > 1 && !scratch) return NTK_E_NULL;
-        a.scratch = scratch;
-    } else {
-        if (dn <= 0 || dv <= 0) return NTK_E_SHAPE;
-        a.kA = K; a.ldA = ldk; a.nA = dn; a.hA = dn;
-        a.v = V; a.ldV = ldv; a.nV = dv; a.hV = dv;
-        a.keyA0 = key0;
-        rows = T;
-        a.splits = 1;
-        a.scratch = nullptr;
-    }
+    a.H = H; a.shared = 0; a.pos0 = pos0; a.T = T; a.window = window; a.scale = scale;
+    a.kA = K; a.ldA = ldk; a.nA = dn; a.hA = dn;
+    a.v = V; a.ldV = ldv; a.nV = dv; a.hV = dv;
+    a.keyA0 = key0;
+    a.splits = 1;
+    a.scratch = nullptr;
+    const int rows = T;
     if (a.nV > 8 * SLAB) return NTK_E_SHAPE;
     const int DKP = (a.nA + a.nB + 3) & ~3;
     const size_t lds = ((size_t)QROWS * DKP + KCH * (SLAB + 1) + QROWS * KCH) * sizeof(float);
     if (lds > 150 * 1024) return NTK_E_SHAPE;
-    hipStream_t s = resolve_stream(stream);
-    const dim3 grid((rows + QROWS - 1) / QROWS, shared ? 1 : H, a.splits);
+    const dim3 grid((rows + QROWS - 1) / QROWS, H, 1);
     if (lds > 48 * 1024) {
         static bool raised = false;   // (idempotent: a race sets the same attribute twice)
         if (!raised) { NTK_HIP_TRY(hipFuncSetAttribute((const void*)latent_attention_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024)); raised = true; }
     }
     hipLaunchKernelGGL(latent_attention_kernel, grid, dim3(256), lds, s, a);
-    int st = last_launch_status();
-    if (st != NTK_OK) return st;
-    if (a.splits > 1) {
-        hipLaunchKernelGGL(latent_attention_merge_kernel, dim3(rows), dim3(64), 0, s, out, ldo, (const float*)scratch, a.splits, a.nV, H);
-        st = last_launch_status();
-    }
-    return st;
+    return last_launch_status();
 }
 
 int ntk_latent_fold_query(float* qf, const float* q, int ldq, const void* w_uk, int wdtype, int T, int H, int dn, int dr, int R, void* stream) {
     if (!qf || !q || !w_uk) return NTK_E_NULL;
     if (T < 0 || H <= 0 || dn <= 0 || dr < 0 || R <= 0) return NTK_E_SHAPE;
     if (T == 0) return NTK_OK;
-    const size_t lds = (size_t)(dn + dr) * sizeof(float);
-    if (wdtype == NTK_DT_BF16) hipLaunchKernelGGL(latent_fold_query_kernel<uint16_t>, dim3(H, T), dim3(256), lds, resolve_stream(stream), qf, q, ldq, (const uint16_t*)w_uk, H, dn, dr, R);
-    else if (wdtype == NTK_DT_F32) hipLaunchKernelGGL(latent_fold_query_kernel<float>, dim3(H, T), dim3(256), lds, resolve_stream(stream), qf, q, ldq, (const float*)w_uk, H, dn, dr, R);
+    const size_t lds = (size_t)(dn + dr + 256) * sizeof(float);
+    const dim3 grid((R + 63) / 64, H, T);
+    if (wdtype == NTK_DT_BF16) hipLaunchKernelGGL(latent_fold_query_kernel<uint16_t>, grid, dim3(256), lds, resolve_stream(stream), qf, q, ldq, (const uint16_t*)w_uk, H, dn, dr, R);
+    else if (wdtype == NTK_DT_F32) hipLaunchKernelGGL(latent_fold_query_kernel<float>, grid, dim3(256), lds, resolve_stream(stream), qf, q, ldq, (const float*)w_uk, H, dn, dr, R);
     else return NTK_E_DTYPE;
     return last_launch_status();
 }
@@ -364,8 +506,9 @@ int ntk_latent_unfold_value(float* out, int ldo, const float* lat, const void* w
     if (T < 0 || H <= 0 || dv <= 0 || R <= 0) return NTK_E_SHAPE;
     if (T == 0) return NTK_OK;
     const size_t lds = (size_t)R * sizeof(float);
-    if (wdtype == NTK_DT_BF16) hipLaunchKernelGGL(latent_unfold_value_kernel<uint16_t>, dim3(H, T), dim3(256), lds, resolve_stream(stream), out, ldo, lat, (const uint16_t*)w_uv, gate, ldg, H, dv, R);
-    else if (wdtype == NTK_DT_F32) hipLaunchKernelGGL(latent_unfold_value_kernel<float>, dim3(H, T), dim3(256), lds, resolve_stream(stream), out, ldo, lat, (const float*)w_uv, gate, ldg, H, dv, R);
+    const dim3 grid((dv + 15) / 16, H, T);
+    if (wdtype == NTK_DT_BF16) hipLaunchKernelGGL(latent_unfold_value_kernel<uint16_t>, grid, dim3(256), lds, resolve_stream(stream), out, ldo, lat, (const uint16_t*)w_uv, gate, ldg, H, dv, R);
+    else if (wdtype == NTK_DT_F32) hipLaunchKernelGGL(latent_unfold_value_kernel<float>, grid, dim3(256), lds, resolve_stream(stream), out, ldo, lat, (const float*)w_uv, gate, ldg, H, dv, R);
     else return NTK_E_DTYPE;
     return last_launch_status();
 }

@@ -11,29 +11,30 @@ namespace ntk {
 
 constexpr int kMaxExperts = 256;
 
-// one wave per token: lanes stride the row, one reduction per expert; lane 0 then does the softmax and the `top` picks
-__global__ __launch_bounds__(256) void moe_route_kernel(int* ids, float* wts, float* sgate, const float* h, int ldh, const float* wr, const float* wsg, int T,
-                                                        int n, int E, int top) {
-    __shared__ float zs[4][kMaxExperts];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int t = blockIdx.x * 4 + wave;
-    if (t >= T) return;
-    const float* x = h + (long long)t * ldh;
-    for (int e = 0; e < E; ++e) {
-        const float* w = wr + (long long)e * n;
+// one workgroup per token: its 16 waves share the experts (wave w: experts w, w + 16, ...), a lane requests its whole part of the router row before
+// it uses any of it; thread 0 then does the softmax and the `top` picks over the scores in LDS
+constexpr int kRouteThreads = 1024;
+__global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(int* ids, float* wts, float* sgate, const float* h, int ldh, const float* wr, const float* wsg,
+                                                                 int n, int E, int top) {
+    __shared__ float z[kMaxExperts];
+    extern __shared__ __attribute__((aligned(16))) float xs[];   // the token's row
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = kRouteThreads / 64;
+    const long long t = blockIdx.x;
+    const float* x = h + t * ldh;
+    for (int k = threadIdx.x; k < n; k += kRouteThreads) xs[k] = x[k];
+    __syncthreads();
+    for (int e = wave; e < E + (wsg ? 1 : 0); e += nw) {
+        const float* w = e < E ? wr + (long long)e * n : wsg;
         float s = 0.0f;
-        for (int k = lane; k < n; k += 64) s = fmaf(w[k], x[k], s);
+        for (int k = lane; k < n; k += 64) s = fmaf(w[k], xs[k], s);
         s = wave_sum(s);
-        if (lane == 0) zs[wave][e] = s;
+        if (lane == 0) {
+            if (e < E) z[e] = s;
+            else if (sgate) sgate[t] = 1.0f / (1.0f + expf(-s));
+        }
     }
-    if (wsg && sgate) {
-        float s = 0.0f;
-        for (int k = lane; k < n; k += 64) s = fmaf(wsg[k], x[k], s);
-        s = wave_sum(s);
-        if (lane == 0) sgate[t] = 1.0f / (1.0f + expf(-s));
-    }
-    if (lane != 0) return;
-    float* z = zs[wave];
+    __syncthreads();
+    if (threadIdx.x != 0) return;
     float m = z[0];
     for (int e = 1; e < E; ++e) m = fmaxf(m, z[e]);
     float den = 0.0f;
@@ -44,33 +45,50 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int* ids, float* wts, fl
         float bv = -1.0f;
         for (int e = 0; e < E; ++e)
             if (z[e] > bv) { bv = z[e]; best = e; }
-        ids[(long long)t * top + s] = best;
+        ids[t * top + s] = best;
         const float sc = bv / den;
-        wts[(long long)t * top + s] = sc;
+        wts[t * top + s] = sc;
         chosen += sc;
         z[best] = -2.0f;
     }
     const float inv = 1.0f / (chosen + 1e-20f);
-    for (int s = 0; s < top; ++s) wts[(long long)t * top + s] *= inv;
+    for (int s = 0; s < top; ++s) wts[t * top + s] *= inv;
 }
 
-// stable counting sort of the pairs by expert, one workgroup: thread e counts, thread 0 scans, thread e places
-__global__ __launch_bounds__(256) void moe_group_kernel(int* offsets, int* order, int* where, const int* ids, int n_pairs, int E) {
-    __shared__ int start[kMaxExperts + 1];
-    const int e = threadIdx.x;
+// Stable counting sort of the pairs by expert, one workgroup of 1024: the pairs are cut into S = 1024 / E' contiguous segments (E' = E rounded up to a
+// power of two), thread (segment, expert) counts its expert in its segment, one scan in (expert, segment) order gives every thread the place of its
+// first row, and it walks its segment once more to place them.  The ids sit in LDS when they fit.
+constexpr int kGroupThreads = 1024, kGroupLdsIds = 24 * 1024;
+__global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(int* offsets, int* order, int* where, const int* ids_g, int n_pairs, int E, int Ep) {
+    __shared__ int cnt[kGroupThreads + 1];
+    __shared__ int ids_s[kGroupLdsIds];
+    const int* ids = ids_g;
+    if (n_pairs <= kGroupLdsIds) {
+        for (int i = threadIdx.x; i < n_pairs; i += kGroupThreads) ids_s[i] = ids_g[i];
+        ids = ids_s;
+    }
+    const int S = kGroupThreads / Ep;
+    const int e = threadIdx.x % Ep, seg = threadIdx.x / Ep;
+    const int per = (n_pairs + S - 1) / S;
+    const int i0 = min(seg * per, n_pairs), i1 = min(i0 + per, n_pairs);
+    __syncthreads();
     int c = 0;
-    if (e < E)
-        for (int i = 0; i < n_pairs; ++i) c += ids[i] == e;
-    if (e < E) start[e + 1] = c;
-    if (e == 0) start[0] = 0;
+    if (e < E && seg < S)
+        for (int i = i0; i < i1; ++i) c += ids[i] == e;
+    // place of thread (e, seg) in (expert, segment) order
+    const int slot = e * S + seg;
+    if (seg < S) cnt[slot] = e < E ? c : 0;
     __syncthreads();
-    if (e == 0)
-        for (int i = 0; i < E; ++i) start[i + 1] += start[i];
+    if (threadIdx.x == 0) {
+        int run = 0;
+        for (int k = 0; k < Ep * S; ++k) { const int v = cnt[k]; cnt[k] = run; run += v; }
+        cnt[Ep * S] = run;
+    }
     __syncthreads();
-    if (e <= E) offsets[e] = start[e];
-    if (e < E) {
-        int at = start[e];
-        for (int i = 0; i < n_pairs; ++i)
+    if (threadIdx.x <= E) offsets[threadIdx.x] = threadIdx.x < E ? cnt[threadIdx.x * S] : cnt[Ep * S];
+    if (e < E && seg < S) {
+        int at = cnt[slot];
+        for (int i = i0; i < i1; ++i)
             if (ids[i] == e) { order[at] = i; where[i] = at; ++at; }
     }
 }
@@ -105,14 +123,17 @@ int ntk_moe_route(int* ids, float* wts, float* sgate, const float* h, int ldh, c
     if (!ids || !wts || !h || !w_router) return NTK_E_NULL;
     if (T < 0 || n <= 0 || E <= 0 || E > kMaxExperts || top <= 0 || top > E || ldh < n) return NTK_E_SHAPE;
     if (T == 0) return NTK_OK;
-    hipLaunchKernelGGL(moe_route_kernel, dim3((T + 3) / 4), dim3(256), 0, resolve_stream(stream), ids, wts, sgate, h, ldh, w_router, shared_gate_w, T, n, E, top);
+    if ((size_t)n * 4 > 128 * 1024) return NTK_E_SHAPE;
+    hipLaunchKernelGGL(moe_route_kernel, dim3(T), dim3(kRouteThreads), (size_t)n * 4, resolve_stream(stream), ids, wts, sgate, h, ldh, w_router, shared_gate_w, n, E, top);
     return last_launch_status();
 }
 
 int ntk_moe_group(int* offsets, int* order, int* where, const int* ids, int T, int top, int E, void* stream) {
     if (!offsets || !order || !where || !ids) return NTK_E_NULL;
     if (T < 0 || top <= 0 || E <= 0 || E >= 256) return NTK_E_SHAPE;
-    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(256), 0, resolve_stream(stream), offsets, order, where, ids, T * top, E);
+    int Ep = 1;
+    while (Ep < E) Ep *= 2;
+    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(kGroupThreads), 0, resolve_stream(stream), offsets, order, where, ids, T * top, E, Ep);
     return last_launch_status();
 }
 

@@ -1,0 +1,106 @@
+"""Seeded synthetic model folders (config.json + model.safetensors, bfloat16) for the layer-list families: the counterpart of the seeded GGUF
+generator (csrc/engine/synth.cpp) for benchmarks that need real-sized layers without a checkpoint.  Values come from one random pool that is
+repeated to fill a tensor -- timing does not care, and gigabytes are written in seconds."""
+from __future__ import annotations
+
+import json
+import math
+import os
+import struct
+from typing import Dict, Tuple
+
+import numpy as np
+
+PRESETS = {
+    # name: width, heads, dim, rot_dim, vdim, kv_rank, q_rank, window, experts, top, ff, shared_ff, vocab
+    "tiny": dict(width=192, heads=4, dim=24, rot_dim=8, vdim=40, kv_rank=64, q_rank=80, window=48, experts=6, top=2, ff=112, shared_ff=160, vocab=1024),
+    "lite": dict(width=2048, heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=768, window=1024, experts=64, top=6, ff=1408, shared_ff=2816, vocab=32000),
+    "mid": dict(width=4096, heads=32, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=1536, window=2048, experts=32, top=4, ff=2048, shared_ff=4096, vocab=64000),
+}
+
+
+def fabolorn_config(preset: str, layers: int = 2, loop_times: int = 1) -> dict:
+    p = PRESETS[preset]
+    ls = []
+    for k in range(layers):
+        windowed = k % 2 == 1
+        mx = {"heads": p["heads"], "dim": p["dim"], "rot_dim": p["rot_dim"], "vdim": p["vdim"], "kv_rank": p["kv_rank"],
+              "scale": 1.0 / math.sqrt(p["dim"] + p["rot_dim"]), "rot": {"base": 1000000.0, "dims": p["rot_dim"]}}
+        if windowed:
+            mx["mask"] = {"size": p["window"]}
+        else:
+            mx["q_rank"] = p["q_rank"]
+            mx["rot"]["scaling"] = {"factor": 8.0, "original": 4096, "fast": 16.0, "slow": 2.0}
+        ml = {"kind": "moe", "expert": {"ff": p["ff"], "limit": 7.0}, "router": {"experts": p["experts"], "top": p["top"]},
+              "shared": {"ff": p["shared_ff"], "limit": 7.0}}
+        ls.append({"type": "latent_attention_2" if windowed else "latent_attention", "mixer": mx, "mlp": ml})
+    cfg = {"architecture": "Fabolorn", "layers": ls, "norm": {"eps": 1e-5}, "vocab": p["vocab"], "width": p["width"]}
+    if loop_times > 1:
+        cfg["loop"] = {"start": 0, "stop": layers, "times": loop_times}
+    return cfg
+
+
+def fabolorn_shapes(cfg: dict) -> Dict[str, Tuple[int, ...]]:
+    W, V = cfg["width"], cfg["vocab"]
+    s: Dict[str, Tuple[int, ...]] = {"embed": (V, W), "final.norm": (W,), "head": (V, W)}
+    if cfg.get("loop"):
+        s["loop.in"] = (W, 2 * W)
+    for i, L in enumerate(cfg["layers"]):
+        p, mx, ml = "l%d." % i, L["mixer"], L.get("mlp")
+        H, dn, dr, dv, R = mx["heads"], mx["dim"], mx["rot_dim"], mx["vdim"], mx["kv_rank"]
+        s[p + "norm1"] = (W,)
+        if "q_rank" in mx:
+            s[p + "mix.dq"], s[p + "mix.dq.norm"], s[p + "mix.uq"] = (mx["q_rank"], W), (mx["q_rank"],), (H * (dn + dr), mx["q_rank"])
+        else:
+            s[p + "mix.q"] = (H * (dn + dr), W)
+        s[p + "mix.dkv"], s[p + "mix.dkv.norm"] = (R + dr, W), (R,)
+        s[p + "mix.uk"], s[p + "mix.uv"], s[p + "mix.g"], s[p + "mix.o"] = (H * dn, R), (H * dv, R), (H * dv, W), (W, H * dv)
+        if ml:
+            s[p + "norm2"] = (W,)
+            ff = ml["expert"]["ff"]
+            for e in range(ml["router"]["experts"]):
+                q = "%smlp.e%d." % (p, e)
+                s[q + "gate"], s[q + "up"], s[q + "down"] = (ff, W), (ff, W), (W, ff)
+            s[p + "mlp.router"] = (ml["router"]["experts"], W)
+            if ml.get("shared"):
+                sf = ml["shared"]["ff"]
+                s[p + "mlp.shared.gate"], s[p + "mlp.shared.up"], s[p + "mlp.shared.down"], s[p + "mlp.shared.sg"] = (sf, W), (sf, W), (W, sf), (1, W)
+    return s
+
+
+def _bf16(a: np.ndarray) -> np.ndarray:
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def write_folder(folder: str, cfg: dict, seed: int = 20260925) -> int:
+    """-> bytes of model.safetensors"""
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    shapes = fabolorn_shapes(cfg)
+    g = np.random.default_rng(seed)
+    pool = g.standard_normal(1 << 22).astype(np.float32)
+    header, at = {}, 0
+    for name, shp in shapes.items():
+        n = int(np.prod(shp)) * 2
+        header[name] = {"dtype": "BF16", "shape": list(shp), "data_offsets": [at, at + n]}
+        at += n
+    hj = json.dumps(header).encode()
+    hj += b" " * (-len(hj) % 8)
+    with open(os.path.join(folder, "model.safetensors"), "wb") as f:
+        f.write(struct.pack("<Q", len(hj)))
+        f.write(hj)
+        for k, (name, shp) in enumerate(shapes.items()):
+            n = int(np.prod(shp))
+            if len(shp) == 1:
+                vals = 0.1 * pool[:n] + (1.0 if name.endswith(".norm") and name != "final.norm" else 0.0)
+                f.write(_bf16(vals).tobytes())
+                continue
+            scale = 1.0 if name == "embed" else 1.0 / math.sqrt(shp[-1])
+            block = _bf16(np.roll(pool, 7919 * k) * scale).tobytes()
+            left = n * 2
+            while left > 0:
+                f.write(block[:min(left, len(block))])
+                left -= len(block)
+    return at

@@ -100,6 +100,21 @@ def test_dense_grouped_and_gathered_rows(dtype, T, top):
     assert rel(y, ref) < (1e-5 if dtype == "float32" else 1e-2)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("T,ff,K", [(1, 20, 40), (3, 37, 64), (8, 160, 96), (6, 1, 24)])
+def test_few_row_product_with_the_clipped_glu_inside(dtype, T, ff, K):
+    """decoding: gate rows, up rows and the activation in one launch == the product followed by the activation"""
+    from ntransformer_amd import layers as Lr
+    g = np.random.default_rng(T + ff)
+    x = (g.standard_normal((T, K)) * 2).astype(np.float32)
+    w = O.bf16_round(torch.tensor(g.standard_normal((2 * ff, K)))).numpy()
+    gu = torch.tensor(x, dtype=O.F) @ torch.tensor(w, dtype=O.F).T
+    gg, uu = gu[:, :ff].clamp(max=1.5), gu[:, ff:].clamp(-1.5, 1.5)
+    ref = gg * torch.sigmoid(1.702 * gg) * (uu + 1.0)
+    assert rel(Lr.dense(x, w, dtype, glu_limit=1.5), ref) < (1e-5 if dtype == "float32" else 1e-2)
+    assert rel(Lr.dense(x, w, dtype, glu_limit=1.5), Lr.clipped_glu(Lr.dense(x, w, dtype), 1.5)) < 1e-6
+
+
 def test_dense_accumulates_onto_start_values():
     from ntransformer_amd import layers as Lr
     g = np.random.default_rng(9)
