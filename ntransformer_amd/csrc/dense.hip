@@ -351,7 +351,7 @@ int ntk_dense(const ntk_dense_desc* d, void* stream) {
         const bool vec = (d->K % 8 == 0) && (d->ldx % 4 == 0) && !((uintptr_t)d->X & 15) && !((uintptr_t)d->W & 15) && (d->wstride % 8 == 0);
         // 128 x 128 tiles where a group has the rows and the launch still fills the chip; 64-row tiles for short groups (experts, short portions)
         const int rows_per_group = d->T / G;
-        const bool big = rows_per_group >= 192 && d->N >= 128 && (long long)((d->T + 127) / 128) * ((d->N + 127) / 128) >= 128;
+        const bool big = rows_per_group >= 192 && d->N >= 128 && (long long)((d->T + 127) / 128) * ((d->N + 127) / 128) >= 224;
         if (big) {
             const dim3 grid((d->N + 127) / 128, (d->T + 127) / 128, G);
             if (vec) hipLaunchKernelGGL((dense_mfma_kernel<128, 128, true>), grid, dim3(256), 0, s, a);

@@ -90,11 +90,12 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(const AttnArgs a)
     const int jlo = a.window > 0 ? max(0, pmin - a.window + 1) : 0;
     const int jhi = pmax;   // inclusive
     // queries into LDS
-    for (int idx = threadIdx.x; idx < QROWS * DKP; idx += 256) {
-        const int i = idx / DKP, d = idx % DKP;
-        float v = 0.0f;
-        if (row0 + i < n_rows_total && d < DK) v = a.q[(long long)row_token(i) * a.ldq + (long long)row_head(i) * DK + d];
-        Qs[idx] = v;
+    for (int d = threadIdx.x; d < DKP; d += 256) {
+        float qv[QROWS];
+#pragma unroll
+        for (int i = 0; i < QROWS; ++i) qv[i] = (row0 + i < n_rows_total && d < DK) ? a.q[(long long)row_token(i) * a.ldq + (long long)row_head(i) * DK + d] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < QROWS; ++i) Qs[i * DKP + d] = qv[i];
     }
     float m[QPW], l[QPW], acc[QPW][8];
     int rpos[QPW];
@@ -118,21 +119,29 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(const AttnArgs a)
         for (int d0 = 0; d0 < DK; d0 += SLAB) {
             const int nd = min(SLAB, DK - d0);
             __syncthreads();
-            for (int idx = threadIdx.x; idx < KCH * SLAB; idx += 256) {
-                const int k = idx / SLAB, d = idx % SLAB;
-                float v = 0.0f;
-                if (k < nk && d < nd) {
-                    const int dd = d0 + d, j = j0 + k;
-                    v = dd < a.nA ? a.kA[(long long)(j - a.keyA0) * a.ldA + (long long)hk * a.hA + dd] : a.kB[(long long)j * a.ldB + (dd - a.nA)];
+            {   // thread -> (key wave + 4 u, entry lane): the sixteen requests of a thread in flight before the first is stored
+                const int d = lane, dd = d0 + d;
+                const bool first = dd < a.nA;
+                const float* src = first ? a.kA + (long long)(j0 - a.keyA0) * a.ldA + (long long)hk * a.hA + dd : a.kB + (long long)j0 * a.ldB + (dd - a.nA);
+                const long long ld = first ? a.ldA : a.ldB;
+                float v[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    const int k = wave + 4 * u;
+                    v[u] = (k < nk && d < nd) ? src[k * ld] : 0.0f;
                 }
-                Sl[k * (SLAB + 1) + d] = v;
+#pragma unroll
+                for (int u = 0; u < 16; ++u) Sl[(wave + 4 * u) * (SLAB + 1) + d] = v[u];
             }
             __syncthreads();
             const float* kr = Sl + lane * (SLAB + 1);
-            for (int d = 0; d < nd; ++d) {
-                const float kvv = kr[d];
+            for (int d = 0; d < nd; d += 4) {      // (entries past nd are zero in the slab, past DK in the queries)
+                const float k0 = kr[d], k1 = kr[d + 1], k2 = kr[d + 2], k3 = kr[d + 3];
 #pragma unroll
-                for (int i = 0; i < QPW; ++i) s[i] = fmaf(Qs[(wave * QPW + i) * DKP + d0 + d], kvv, s[i]);
+                for (int i = 0; i < QPW; ++i) {
+                    const float4 q4 = *reinterpret_cast<const float4*>(Qs + (wave * QPW + i) * DKP + d0 + d);
+                    s[i] = fmaf(q4.x, k0, s[i]); s[i] = fmaf(q4.y, k1, s[i]); s[i] = fmaf(q4.z, k2, s[i]); s[i] = fmaf(q4.w, k3, s[i]);
+                }
             }
         }
         // ---- online softmax, weights to LDS
@@ -159,17 +168,26 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(const AttnArgs a)
             if (v0 < a.nV) {
                 const int nvv = min(SLAB, a.nV - v0);
                 __syncthreads();
-                for (int idx = threadIdx.x; idx < KCH * SLAB; idx += 256) {
-                    const int k = idx / SLAB, d = idx % SLAB;
-                    float v = 0.0f;
-                    if (k < nk && d < nvv) v = a.v[(long long)(j0 + k - a.keyA0) * a.ldV + (long long)hv * a.hV + v0 + d];
-                    Sl[k * SLAB + d] = v;
+                {
+                    const float* src = a.v + (long long)(j0 - a.keyA0) * a.ldV + (long long)hv * a.hV + v0 + lane;
+                    float v[16];
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) {
+                        const int k = wave + 4 * u;
+                        v[u] = (k < nk && lane < nvv) ? src[k * a.ldV] : 0.0f;
+                    }
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) Sl[(wave + 4 * u) * SLAB + lane] = v[u];
                 }
                 __syncthreads();
-                for (int k = 0; k < nk; ++k) {
-                    const float vv = Sl[k * SLAB + lane];
+                for (int k = 0; k < nk; k += 4) {      // (weights and value rows past nk are zero)
+                    const float x0 = Sl[k * SLAB + lane], x1 = Sl[(k + 1) * SLAB + lane], x2 = Sl[(k + 2) * SLAB + lane], x3 = Sl[(k + 3) * SLAB + lane];
 #pragma unroll
-                    for (int i = 0; i < QPW; ++i) acc[i][c] = fmaf(Ps[(wave * QPW + i) * KCH + k], vv, acc[i][c]);
+                    for (int i = 0; i < QPW; ++i) {
+                        const float4 p4 = *reinterpret_cast<const float4*>(Ps + (wave * QPW + i) * KCH + k);
+                        acc[i][c] = fmaf(p4.x, x0, acc[i][c]); acc[i][c] = fmaf(p4.y, x1, acc[i][c]);
+                        acc[i][c] = fmaf(p4.z, x2, acc[i][c]); acc[i][c] = fmaf(p4.w, x3, acc[i][c]);
+                    }
                 }
             }
         }
@@ -225,11 +243,18 @@ __global__ __launch_bounds__(256) void latent_attention_shared_kernel(const Shar
     const int last_row = min(row0 + SROWS, n_rows) - 1;
     const int pmin = a.pos0 + row0 / a.H, pmax = a.pos0 + last_row / a.H;
     const int jlo = a.window > 0 ? max(0, pmin - a.window + 1) : 0, jhi = pmax;
-    for (int idx = tid; idx < SROWS * DKP; idx += 256) {
-        const int i = idx / DKP, d = idx % DKP, r = row0 + i;
-        Qs[idx] = (r < n_rows && d < DK) ? a.q[(long long)(r / a.H) * a.ldq + (long long)(r % a.H) * DK + d] : 0.0f;
+    for (int d = tid; d < DKP; d += 256) {          // the 16 query rows: all requests of a pass in flight before the first is stored
+        float qv[SROWS];
+#pragma unroll
+        for (int i = 0; i < SROWS; ++i) {
+            const int r = row0 + i;
+            qv[i] = (r < n_rows && d < DK) ? a.q[(long long)(r / a.H) * a.ldq + (long long)(r % a.H) * DK + d] : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < SROWS; ++i) Qs[i * DKP + d] = qv[i];
     }
     if (tid < SROWS) { ms[tid] = -INFINITY; ls[tid] = 0.0f; }
+    const int lane = tid & 63, wave = tid >> 6;
     const int key = tid % KB, rg = tid / KB;       // scores: rows 2 rg, 2 rg + 1
     const int rpos0 = row0 + 2 * rg < n_rows ? a.pos0 + (row0 + 2 * rg) / a.H : -1;
     const int rpos1 = row0 + 2 * rg + 1 < n_rows ? a.pos0 + (row0 + 2 * rg + 1) / a.H : -1;
@@ -245,19 +270,27 @@ __global__ __launch_bounds__(256) void latent_attention_shared_kernel(const Shar
         if (tile % a.splits != (int)blockIdx.y) continue;
         const int nk = min(KB, jhi + 1 - j0);
         __syncthreads();                           // the previous tile is used up (and Qs / ms are written)
-        if (vec4) {
-            const int q4 = DK / 4;
-            for (int idx = tid; idx < KB * q4; idx += 256) {
-                const int k = idx / q4, c4 = idx % q4;
-                float4 v = float4{0.f, 0.f, 0.f, 0.f};
-                if (k < nk) v = *reinterpret_cast<const float4*>(a.cache + (long long)(j0 + k) * a.row + 4 * c4);
-                *reinterpret_cast<float4*>(Ks + k * DKP + 4 * c4) = v;
+        if (vec4) {                                // 16 bytes per request, eight requests of a thread in flight before the first is stored
+            const int q4 = DK / 4, total = KB * q4, dk = 256 / q4, dc = 256 % q4;
+            int k = tid / q4, c = tid % q4;
+            for (int base = tid; base < total; base += 256 * 8) {
+                float4 v[8];
+                int at[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    at[u] = k * DKP + 4 * c;
+                    v[u] = float4{0.f, 0.f, 0.f, 0.f};
+                    if (base + 256 * u < total && k < nk) v[u] = *reinterpret_cast<const float4*>(a.cache + (long long)(j0 + k) * a.row + 4 * c);
+                    c += dc; k += dk;
+                    if (c >= q4) { c -= q4; ++k; }
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    if (base + 256 * u < total) *reinterpret_cast<float4*>(Ks + at[u]) = v[u];
             }
         } else {
-            for (int idx = tid; idx < KB * DKP; idx += 256) {
-                const int k = idx / DKP, d = idx % DKP;
-                Ks[idx] = (k < nk && d < DK) ? a.cache[(long long)(j0 + k) * a.row + d] : 0.0f;
-            }
+            for (int k = wave; k < KB; k += 4)
+                for (int d = lane; d < DKP; d += 64) Ks[k * DKP + d] = (k < nk && d < DK) ? a.cache[(long long)(j0 + k) * a.row + d] : 0.0f;
         }
         __syncthreads();
         // ---- scores
@@ -276,18 +309,29 @@ __global__ __launch_bounds__(256) void latent_attention_shared_kernel(const Shar
         Ps[(2 * rg) * KB + key] = v0 ? s0 * a.scale : -INFINITY;
         Ps[(2 * rg + 1) * KB + key] = v1 ? s1 * a.scale : -INFINITY;
         __syncthreads();
-        // ---- online softmax, one thread per row
-        if (tid < SROWS) {
-            float* p = Ps + tid * KB;
-            float mc = -INFINITY;
-            for (int k = 0; k < KB; ++k) mc = fmaxf(mc, p[k]);
-            const float mn = fmaxf(ms[tid], mc), msafe = mn == -INFINITY ? 0.0f : mn;
-            const float corr = ms[tid] == -INFINITY ? 0.0f : expf(ms[tid] - msafe);
-            float sum = 0.0f;
-            for (int k = 0; k < KB; ++k) { const float e = p[k] == -INFINITY ? 0.0f : expf(p[k] - msafe); p[k] = e; sum += e; }
-            ls[tid] = ls[tid] * corr + sum;
-            ms[tid] = mn;
-            cr[tid] = corr;
+        // ---- online softmax: 16 lanes per row, two keys each
+        {
+            const int row = tid >> 4, sub = tid & 15;
+            float* p = Ps + row * KB;
+            const float a0 = p[sub], a1 = p[sub + 16];
+            float mc = fmaxf(a0, a1);
+#pragma unroll
+            for (int o = 8; o >= 1; o >>= 1) mc = fmaxf(mc, __shfl_xor(mc, o, 16));
+            const float mo = ms[row];
+            const float mn = fmaxf(mo, mc), msafe = mn == -INFINITY ? 0.0f : mn;
+            const float e0 = a0 == -INFINITY ? 0.0f : expf(a0 - msafe), e1 = a1 == -INFINITY ? 0.0f : expf(a1 - msafe);
+            float sum = e0 + e1;
+#pragma unroll
+            for (int o = 8; o >= 1; o >>= 1) sum += __shfl_xor(sum, o, 16);
+            p[sub] = e0;
+            p[sub + 16] = e1;
+            __syncthreads();                       // every lane has read ms[row]
+            if (sub == 0) {
+                const float corr = mo == -INFINITY ? 0.0f : expf(mo - msafe);
+                ls[row] = ls[row] * corr + sum;
+                ms[row] = mn;
+                cr[row] = corr;
+            }
         }
         __syncthreads();
         // ---- weighted latents: thread -> column tid (+ 256)
@@ -310,13 +354,15 @@ __global__ __launch_bounds__(256) void latent_attention_shared_kernel(const Shar
         }
     }
     __syncthreads();
-    for (int i = 0; i < SROWS; ++i) {
-        if (row0 + i >= n_rows) break;
-        float* st = a.scratch + ((long long)(row0 + i) * a.splits + blockIdx.y) * (2 + a.R);
-        if (tid == 0) { st[0] = ms[i]; st[1] = ls[i]; }
 #pragma unroll
-        for (int c = 0; c < RC; ++c)
-            if (tid + 256 * c < a.R) st[2 + tid + 256 * c] = acc[c][i];
+    for (int i = 0; i < SROWS; ++i) {              // (unrolled: the sums stay in registers)
+        if (row0 + i < n_rows) {
+            float* st = a.scratch + ((long long)(row0 + i) * a.splits + blockIdx.y) * (2 + a.R);
+            if (tid == 0) { st[0] = ms[i]; st[1] = ls[i]; }
+#pragma unroll
+            for (int c = 0; c < RC; ++c)
+                if (tid + 256 * c < a.R) st[2 + tid + 256 * c] = acc[c][i];
+        }
     }
 }
 

@@ -23,10 +23,19 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(int* ids, floa
     const float* x = h + t * ldh;
     for (int k = threadIdx.x; k < n; k += kRouteThreads) xs[k] = x[k];
     __syncthreads();
+    const bool vec = (n % 4 == 0) && !((uintptr_t)wr & 15) && !(wsg && ((uintptr_t)wsg & 15));
     for (int e = wave; e < E + (wsg ? 1 : 0); e += nw) {
         const float* w = e < E ? wr + (long long)e * n : wsg;
         float s = 0.0f;
-        for (int k = lane; k < n; k += 64) s = fmaf(w[k], xs[k], s);
+        if (vec) {
+#pragma unroll 4
+            for (int k = lane * 4; k < n; k += 256) {
+                const float4 a4 = *reinterpret_cast<const float4*>(w + k), x4 = *reinterpret_cast<const float4*>(xs + k);
+                s = fmaf(a4.x, x4.x, s); s = fmaf(a4.y, x4.y, s); s = fmaf(a4.z, x4.z, s); s = fmaf(a4.w, x4.w, s);
+            }
+        } else {
+            for (int k = lane; k < n; k += 64) s = fmaf(w[k], xs[k], s);
+        }
         s = wave_sum(s);
         if (lane == 0) {
             if (e < E) z[e] = s;
@@ -34,25 +43,39 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(int* ids, floa
         }
     }
     __syncthreads();
-    if (threadIdx.x != 0) return;
-    float m = z[0];
-    for (int e = 1; e < E; ++e) m = fmaxf(m, z[e]);
+    if (wave != 0) return;
+    // softmax and the picks by one wave: lane l holds experts l, l + 64, l + 128, l + 192
+    float v[4];
+    float m = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) { v[c] = lane + 64 * c < E ? z[lane + 64 * c] : -INFINITY; m = fmaxf(m, v[c]); }
+    m = wave_max(m);
     float den = 0.0f;
-    for (int e = 0; e < E; ++e) { z[e] = expf(z[e] - m); den += z[e]; }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) { v[c] = lane + 64 * c < E ? expf(v[c] - m) : -1.0f; den += fmaxf(v[c], 0.0f); }
+    den = wave_sum(den);
+    __shared__ int pick_id[kMaxExperts];
+    __shared__ float pick_sc[kMaxExperts];
     float chosen = 0.0f;
     for (int s = 0; s < top; ++s) {
-        int best = -1;
-        float bv = -1.0f;
-        for (int e = 0; e < E; ++e)
-            if (z[e] > bv) { bv = z[e]; best = e; }
-        ids[t * top + s] = best;
+        float bv = v[0];
+        int bi = lane;
+#pragma unroll
+        for (int c = 1; c < 4; ++c)
+            if (v[c] > bv) { bv = v[c]; bi = lane + 64 * c; }      // (equal values: the lower index stays)
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) {
+            const float ov = __shfl_xor(bv, o, 64);
+            const int oi = __shfl_xor(bi, o, 64);
+            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        }
         const float sc = bv / den;
-        wts[t * top + s] = sc;
         chosen += sc;
-        z[best] = -2.0f;
+        if (lane == 0) { pick_id[s] = bi; pick_sc[s] = sc; }
+        if ((bi & 63) == lane) v[bi >> 6] = -2.0f;
     }
     const float inv = 1.0f / (chosen + 1e-20f);
-    for (int s = 0; s < top; ++s) wts[t * top + s] *= inv;
+    for (int s = lane; s < top; s += 64) { ids[t * top + s] = pick_id[s]; wts[t * top + s] = pick_sc[s] * inv; }   // (same wave wrote them: in order)
 }
 
 // Stable counting sort of the pairs by expert, one workgroup of 1024: the pairs are cut into S = 1024 / E' contiguous segments (E' = E rounded up to a
