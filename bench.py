@@ -64,6 +64,7 @@ def parse():
                     help="instead of the default workload: prompt and decode throughput of a layer-list family on synthetic real-sized layers, beside the "
                          "Llama path at equal width / heads / active feed-forward width (F16 and Q8_0); one JSON line of its own")
     ap.add_argument("--family-size", default="lite", choices=["tiny", "lite", "mid"])
+    ap.add_argument("--family-no-compare", action="store_true", help="skip the Llama runs beside the family (a profile of the family's kernels alone)")
     ap.add_argument("--family-layers", type=int, default=2)
     ap.add_argument("--family-dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prompt-bench", type=int, default=1024, help="also time one prompt pass of this many tokens (0 = skip); reported under config.prompt_pass")
@@ -429,7 +430,7 @@ def run_family(args):
         eng.close()
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
-    for mix in ("F16", "Q8_0"):
+    for mix in (() if args.family_no_compare else ("F16", "Q8_0")):
         try:
             inter = p["top"] * p["ff"] + p["shared_ff"]
             inter -= inter % 256

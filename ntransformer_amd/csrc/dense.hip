@@ -247,6 +247,7 @@ __global__ __launch_bounds__(256) void dense_gemv_kernel(const DenseArgs a) {
 #pragma unroll
     for (int i = 0; i < RW; ++i) s[i] = 0.0f;
     if (a.vec) {
+#pragma unroll 2
         for (int k = lane * 8; k < a.K; k += 64 * 8) {
             float wv[RW][8];
             if constexpr (sizeof(WT) == 2) {

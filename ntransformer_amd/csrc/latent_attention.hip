@@ -6,9 +6,9 @@
 //   * shared (few query tokens, decoding): the query's unrotated part is folded through the key up-projection first (ntk_latent_fold_query), so every
 //     head scores against the cache rows themselves, [c | rotated] . [folded q | rotated q]; the weighted sum is taken over c and the value
 //     up-projection is applied once afterwards (ntk_latent_unfold_value).  Nothing per head is ever materialised for the cached positions.
-// Both are one kernel: a workgroup owns 16 query rows (tokens of one head / (token, head) pairs) and walks the visible keys in chunks of 64:
-// lane = key for the scores (key slab of 64 dims at a time in LDS), online softmax per row in F32, lane = value column for the weighted sum.
-// With splits > 1 the chunks go round the splits and a second launch merges the partial (max, sum, vector) states.
+// Expanded: a workgroup owns 16 tokens of one head and walks the visible keys in chunks of 64 -- lane = key for the scores (key slabs of 64 entries in
+// LDS), online softmax per row in F32, lane = value column for the weighted sum.  Shared: a workgroup owns 16 (token, head) rows and whole tiles of 32
+// cache rows; the tiles go round up to 128 workgroups and a second launch merges their (max, sum, vector) states.
 #include "common.hip.h"
 #include "../../include/ntk_layers.h"
 
@@ -63,9 +63,8 @@ struct AttnArgs {
     const float* kB; long long ldB; int nB;           // second part: kB + j * ldB, nB entries (the rotated part inside the cache row)
     const float* v; long long ldV; int nV; int hV;    // value: v + (j - keyA0) * ldV + h * hV
     int keyA0;
-    int H, shared, pos0, T, window;
+    int H, pos0, T, window;
     float scale;
-    int splits; float* scratch;       // splits > 1: partial states [row][split][2 + nV]
 };
 
 constexpr int QROWS = 16, QPW = 4, KCH = 64, SLAB = 64;
@@ -79,14 +78,13 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(const AttnArgs a)
     float* Ps = Sl + KCH * (SLAB + 1);             // [QROWS][KCH]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     // rows of this workgroup
-    int head, n_rows_total;
-    if (a.shared) { head = 0; n_rows_total = a.T * a.H; } else { head = blockIdx.y; n_rows_total = a.T; }
+    const int head = blockIdx.y, n_rows_total = a.T;   // rows = the tokens of this portion, for one head
     const int row0 = blockIdx.x * QROWS;
-    auto row_token = [&](int i) { const int r = row0 + i; return a.shared ? r / a.H : r; };
-    auto row_head = [&](int i) { const int r = row0 + i; return a.shared ? r % a.H : head; };
+    auto row_token = [&](int i) { return row0 + i; };
+    auto row_head = [&](int) { return head; };
     const int last_row = min(row0 + QROWS, n_rows_total) - 1;
-    const int pmin = a.pos0 + (a.shared ? row0 / a.H : row0);
-    const int pmax = a.pos0 + (a.shared ? last_row / a.H : last_row);
+    const int pmin = a.pos0 + row0;
+    const int pmax = a.pos0 + last_row;
     const int jlo = a.window > 0 ? max(0, pmin - a.window + 1) : 0;
     const int jhi = pmax;   // inclusive
     // queries into LDS
@@ -107,10 +105,8 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(const AttnArgs a)
 #pragma unroll
         for (int c = 0; c < 8; ++c) acc[i][c] = 0.0f;
     }
-    const int hk = a.shared ? 0 : head;
-    int chunk = 0;
-    for (int j0 = jlo; j0 <= jhi; j0 += KCH, ++chunk) {
-        if (a.splits > 1 && chunk % a.splits != (int)blockIdx.z) continue;
+    const int hk = head;
+    for (int j0 = jlo; j0 <= jhi; j0 += KCH) {
         const int nk = min(KCH, jhi + 1 - j0);
         float s[QPW];
 #pragma unroll
@@ -161,7 +157,7 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(const AttnArgs a)
             Ps[(wave * QPW + i) * KCH + lane] = p;
         }
         // ---- weighted sum: slabs of SLAB value columns, lane = column
-        const int hv = a.shared ? 0 : head;
+        const int hv = head;
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
             const int v0 = c * SLAB;
@@ -198,19 +194,11 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(const AttnArgs a)
         const int ri = wave * QPW + i;
         if (row0 + ri >= n_rows_total) continue;
         const int t = row_token(ri), h = row_head(ri);
-        if (a.splits > 1) {
-            float* st = a.scratch + ((long long)(row0 + ri) * a.splits + blockIdx.z) * (2 + a.nV);   // (splits only in the shared form: row = t * H + h)
-            if (lane == 0) { st[0] = m[i]; st[1] = l[i]; }
+        const float inv = l[i] > 0.0f ? 1.0f / l[i] : 0.0f;
+        float* o = a.out + (long long)t * a.ldo + (long long)h * a.nV;
 #pragma unroll
-            for (int c = 0; c < 8; ++c)
-                if (c * SLAB + lane < a.nV) st[2 + c * SLAB + lane] = acc[i][c];
-        } else {
-            const float inv = l[i] > 0.0f ? 1.0f / l[i] : 0.0f;
-            float* o = a.out + (long long)t * a.ldo + (long long)h * a.nV;
-#pragma unroll
-            for (int c = 0; c < 8; ++c)
-                if (c * SLAB + lane < a.nV) o[c * SLAB + lane] = acc[i][c] * inv;
-        }
+        for (int c = 0; c < 8; ++c)
+            if (c * SLAB + lane < a.nV) o[c * SLAB + lane] = acc[i][c] * inv;
     }
 }
 
@@ -514,12 +502,10 @@ int ntk_latent_attention(float* out, int ldo, const float* q, int ldq, const flo
     AttnArgs a{};
     a.out = out; a.ldo = ldo; a.q = q; a.ldq = ldq;
     a.kB = cache + kv_rank; a.ldB = row; a.nB = rot_dim;
-    a.H = H; a.shared = 0; a.pos0 = pos0; a.T = T; a.window = window; a.scale = scale;
+    a.H = H; a.pos0 = pos0; a.T = T; a.window = window; a.scale = scale;
     a.kA = K; a.ldA = ldk; a.nA = dn; a.hA = dn;
     a.v = V; a.ldV = ldv; a.nV = dv; a.hV = dv;
     a.keyA0 = key0;
-    a.splits = 1;
-    a.scratch = nullptr;
     const int rows = T;
     if (a.nV > 8 * SLAB) return NTK_E_SHAPE;
     const int DKP = (a.nA + a.nB + 3) & ~3;

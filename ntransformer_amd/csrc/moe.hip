@@ -100,15 +100,27 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(int* offsets, 
         for (int i = i0; i < i1; ++i) c += ids[i] == e;
     // place of thread (e, seg) in (expert, segment) order
     const int slot = e * S + seg;
-    if (seg < S) cnt[slot] = e < E ? c : 0;
+    cnt[slot] = e < E ? c : 0;             // Ep * S = 1024: every thread has a slot
     __syncthreads();
-    if (threadIdx.x == 0) {
-        int run = 0;
-        for (int k = 0; k < Ep * S; ++k) { const int v = cnt[k]; cnt[k] = run; run += v; }
-        cnt[Ep * S] = run;
+    {   // exclusive scan of the Ep * S (= 1024) counts: inside each wave by shuffles, the 16 wave totals by the first lanes
+        __shared__ int wave_total[kGroupThreads / 64];
+        const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+        const int mine = cnt[threadIdx.x];
+        int inc = mine;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int up = __shfl_up(inc, o, 64);
+            if (lane >= o) inc += up;
+        }
+        if (lane == 63) wave_total[wv] = inc;
+        __syncthreads();
+        int before = 0;
+        for (int k = 0; k < wv; ++k) before += wave_total[k];
+        cnt[threadIdx.x] = before + inc - mine;
+        if (threadIdx.x == kGroupThreads - 1) cnt[kGroupThreads] = before + inc;
     }
     __syncthreads();
-    if (threadIdx.x <= E) offsets[threadIdx.x] = threadIdx.x < E ? cnt[threadIdx.x * S] : cnt[Ep * S];
+    if (threadIdx.x <= E) offsets[threadIdx.x] = threadIdx.x < E ? cnt[threadIdx.x * S] : cnt[kGroupThreads];
     if (e < E && seg < S) {
         int at = cnt[slot];
         for (int i = i0; i < i1; ++i)
