@@ -162,6 +162,10 @@ int64_t nt_synth_tensor(const nt_synth_spec* spec, const char* name, void* dst, 
  * use them without a device. */
 /* JSON description of a GGUF file: config, tensor table, vocab size. Returns bytes needed (excl. NUL) or negative. */
 int   nt_gguf_describe(const char* path, char* json_out, int cap);
+/* JSON description of a model FOLDER (config.json + model.safetensors): architecture, whether a family for it is built in, the families that are,
+ * the tensor table (name, dtype, shape, bytes).  Returns bytes needed (excl. NUL) or a negative NTK_E_* (unreadable, malformed header, offsets that
+ * do not fit a tensor's shape or the file). */
+int   nt_model_folder_describe(const char* path, char* json_out, int cap);
 typedef void* nt_tokenizer_t;
 nt_tokenizer_t nt_tokenizer_open(const char* gguf_path);       /* NULL on failure */
 void  nt_tokenizer_close(nt_tokenizer_t t);

@@ -3,6 +3,7 @@
 #include "../../../include/ntransformer.h"
 #include "../../../include/ntk_engine.h"
 #include "engine.h"
+#include "safetensors.h"
 
 #include <cstdlib>
 #include <cstring>
@@ -284,6 +285,40 @@ static void json_escape(std::string& o, const std::string& s) {
         else if (c < 0x20) { char b[8]; snprintf(b, sizeof b, "\\u%04x", c); o += b; }
         else o.push_back((char)c);
     }
+}
+
+// host only: what a model folder holds (config's architecture, whether a family for it is built in, the tensor table) as JSON
+int nt_model_folder_describe(const char* path, char* out, int cap) {
+    if (!path) return NTK_E_NULL;
+    try {
+        nt::ModelFolder f;
+        const int st = f.open(path);
+        if (st != NTK_OK) return st;
+        const std::string arch = f.config().at("architecture").str;
+        bool known = false;
+        std::string fams;
+        for (const auto& n : nt::registered_families()) { known = known || n == arch; fams += (fams.empty() ? "\"" : ",\"") + n + "\""; }
+        std::string j = "{\"architecture\":\"";
+        json_escape(j, arch);
+        j += std::string("\",\"family_built_in\":") + (known ? "true" : "false") + ",\"families\":[" + fams + "],\"tensors\":[";
+        bool first = true;
+        size_t total = 0;
+        for (const auto& kv : f.tensors()) {
+            if (!first) j += ",";
+            first = false;
+            j += "{\"name\":\""; json_escape(j, kv.first); j += "\",\"dtype\":\""; json_escape(j, kv.second.dtype); j += "\",\"shape\":[";
+            for (size_t d = 0; d < kv.second.shape.size(); ++d) { if (d) j += ","; j += std::to_string(kv.second.shape[d]); }
+            j += "],\"nbytes\":" + std::to_string(kv.second.nbytes) + "}";
+            total += kv.second.nbytes;
+        }
+        j += "],\"tensor_bytes\":" + std::to_string(total) + "}";
+        if (out && cap > 0) {
+            const size_t k = std::min<size_t>(j.size(), (size_t)cap - 1);
+            memcpy(out, j.data(), k);
+            out[k] = 0;
+        }
+        return (int)j.size();
+    } catch (...) { return NTK_E_NOMEM; }
 }
 
 int nt_gguf_describe(const char* path, char* out, int cap) {
