@@ -37,6 +37,9 @@ typedef struct ntk_dense_desc {
     /* glu_ff > 0 (only with T <= ntk_dense_few_rows(), N == 2 * glu_ff, no accumulate): W holds glu_ff gate rows then glu_ff up rows and
      * Y[r][f] = g' * sigmoid(glu_alpha * g') * (u' + 1), g' = min(gate, glu_limit), u' = clamp(up, -glu_limit, glu_limit) -- the product and ntk_clipped_glu in one launch */
     int glu_ff; float glu_limit, glu_alpha;
+    /* norm_w != NULL (only with T <= ntk_dense_few_rows()): every activation row is first divided by sqrt(mean(x^2) + norm_eps) and multiplied by
+     * (norm_offset + norm_w[k]), norm_w F32 [K] -- ntk_rmsnorm_offset and the product in one launch */
+    const float* norm_w; float norm_eps, norm_offset;
 } ntk_dense_desc;
 int ntk_dense_few_rows(void);   /* up to this many rows a product takes the row-streaming form */
 int ntk_dense(const ntk_dense_desc* d, void* stream);

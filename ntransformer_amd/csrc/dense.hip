@@ -33,6 +33,7 @@ struct DenseArgs {
     const int* rows; int row_div;
     int T, N, K, accumulate, G, vec;
     int glu_ff; float glu_limit, glu_alpha;   // few-row form only: outputs f < glu_ff = clipped GLU of rows f (gate) and glu_ff + f (up)
+    const float* norm_w; float norm_eps, norm_offset;   // few-row form only: the activation row is RMS-normed with weight (offset + norm_w) first
 };
 
 __device__ __forceinline__ bool group_range(const DenseArgs& a, int g, int& r0, int& r1) {
@@ -228,7 +229,14 @@ __global__ __launch_bounds__(256) void dense_gemv_kernel(const DenseArgs a) {
         while (r >= a.offsets[g + 1]) ++g;
     }
     const float* xrow = a.X + (long long)(a.rows ? a.rows[r] / a.row_div : r) * a.ldx;
-    for (int k = threadIdx.x; k < a.K; k += 256) xs[k] = xrow[k];
+    float ss = 0.0f;
+    for (int k = threadIdx.x; k < a.K; k += 256) { const float v = xrow[k]; xs[k] = v; ss = fmaf(v, v, ss); }
+    if (a.norm_w) {                                         // (uniform over the launch)
+        __shared__ float red[16];
+        ss = block_sum(ss, red);
+        const float inv = 1.0f / sqrtf(ss / (float)a.K + a.norm_eps);
+        for (int k = threadIdx.x; k < a.K; k += 256) xs[k] = xs[k] * inv * (a.norm_offset + a.norm_w[k]);   // (each thread rewrites what it wrote)
+    }
     __syncthreads();
     const WT* W = (const WT*)a.W + (long long)g * a.wstride;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -336,13 +344,15 @@ int ntk_dense(const ntk_dense_desc* d, void* stream) {
     if (d->offsets && d->G <= 0) return NTK_E_SHAPE;
     if (d->rows && d->row_div <= 0) return NTK_E_SHAPE;
     if (d->glu_ff > 0 && (d->T > kGemvRows || d->N != 2 * d->glu_ff || d->accumulate)) return NTK_E_SHAPE;
+    if (d->norm_w && d->T > kGemvRows) return NTK_E_SHAPE;
     if (d->T == 0) return NTK_OK;
     const int G = d->offsets ? d->G : 1;
-    DenseArgs a{d->Y, d->ldy, d->X, d->ldx, d->W, d->wstride, d->offsets, d->rows, d->rows ? d->row_div : 1, d->T, d->N, d->K, d->accumulate, G, 0, 0, 0.0f, 0.0f};
+    DenseArgs a{d->Y, d->ldy, d->X, d->ldx, d->W, d->wstride, d->offsets, d->rows, d->rows ? d->row_div : 1, d->T, d->N, d->K, d->accumulate, G, 0, 0, 0.0f, 0.0f, nullptr, 0.0f, 0.0f};
     hipStream_t s = resolve_stream(stream);
     if (d->T <= kGemvRows) {
         if ((size_t)d->K * 4 > 160 * 1024 - 1024) return NTK_E_SHAPE;
         a.glu_ff = d->glu_ff; a.glu_limit = d->glu_limit; a.glu_alpha = d->glu_alpha;
+        a.norm_w = d->norm_w; a.norm_eps = d->norm_eps; a.norm_offset = d->norm_offset;
         a.vec = (d->K % 8 == 0) && !((uintptr_t)d->W & 15) && !((d->wstride * (d->wdtype == NTK_DT_BF16 ? 2 : 4)) & 15);
         if (d->wdtype == NTK_DT_BF16) launch_gemv<uint16_t>(a, d->T, s);
         else launch_gemv<float>(a, d->T, s);

@@ -21,6 +21,7 @@ LayerStackModel::~LayerStackModel() {
     for (void* p : allocs_) nt_hip_free(p);
     if (logits_) nt_hip_free(logits_);
     if (capture_buf_) nt_hip_free(capture_buf_);
+    if (h_stage_) nt_hip_free_host(h_stage_);
 }
 
 void* LayerStackModel::dev_alloc(size_t bytes) {
@@ -298,7 +299,10 @@ int LayerStackModel::alloc_buffers() {
     bool ok = fl(&x_, C * W) && fl(&x0_, C * W) && fl(&cat_, C * 2 * W) && fl(&h1_, C * W) && fl(&h2_, C * W) && fl(&a_, C * max_in_) &&
               fl(&cq_, C * std::max(max_qrank_, 1)) && fl(&q_, C * max_hqd_) && fl(&qf_, (size_t)kSharedRows * max_fold_) && fl(&lat_, (size_t)kSharedRows * max_hr_) &&
               fl(&att_, C * max_hdv_) && fl(&kx_, ctx * max_hdn_) && fl(&vx_, ctx * max_hdv_) && fl(&mix_, C * W) && fl(&xw_, C * W) && fl(&hn_, C * W) &&
-              in(&tokens_dev_, C) && in(&want_dev_, C);
+              in(&tokens_dev_, 2 * C);
+    want_dev_ = tokens_dev_ ? tokens_dev_ + C : nullptr;   // one staging area: [tokens of a pass | wanted places], filled by ONE stream-ordered copy from pinned memory
+    h_stage_ = (int*)nt_hip_malloc_host(2 * C * sizeof(int));
+    ok = ok && h_stage_ != nullptr;
     size_t sc = 0;
     for (const auto& L : layers_) sc = std::max(sc, ntk_latent_attention_scratch(kSharedRows, L.mix.heads, L.mix.kv_rank, opt_.max_context));
     ok = ok && fl(&scratch_, sc);
@@ -330,13 +334,19 @@ int LayerStackModel::truncate_slot(int slot, int length) {
 int LayerStackModel::run_mixer(const StackLayer& L, float* cache, int T, int pos0) {
     const LatentMixer& m = L.mix;
     const int W = info_.width, H = m.heads, qd = m.qd(), row = m.row(), hv = H * m.vdim, na = (int)m.in.out_f;
-    // one product for [query (latent) | latent + key part | gate]
-    LS_TRY(ntk_dense_linear(a_, na, h1_, W, m.in.ptr, m.in.dtype, T, na, W, 0, stream_));
+    // one product for [query (latent) | latent + key part | gate]; decoding: the layer's first norm and the query latent's norm run inside the products
+    const bool few = T <= ntk_dense_few_rows();
+    ntk_dense_desc d{};
+    d.Y = a_; d.ldy = na; d.X = few ? x_ : h1_; d.ldx = W; d.W = m.in.ptr; d.wdtype = m.in.dtype; d.G = 1; d.row_div = 1; d.T = T; d.N = na; d.K = W;
+    if (few) { d.norm_w = L.norm1; d.norm_eps = eps_; d.norm_offset = 1.0f; }
+    LS_TRY(ntk_dense(&d, stream_));
     float* q = a_;
     int ldq = na;
     if (m.q_rank) {
-        LS_TRY(ntk_rmsnorm_offset(cq_, m.q_norm, nullptr, nullptr, m.q_rank, a_, na, T, m.q_rank, eps_, 0.0f, stream_));
-        LS_TRY(ntk_dense_linear(q_, H * qd, cq_, m.q_rank, m.uq.ptr, m.uq.dtype, T, H * qd, m.q_rank, 0, stream_));
+        d.Y = q_; d.ldy = H * qd; d.X = few ? a_ : cq_; d.ldx = few ? na : m.q_rank; d.W = m.uq.ptr; d.wdtype = m.uq.dtype; d.N = H * qd; d.K = m.q_rank;
+        if (few) { d.norm_w = m.q_norm; d.norm_offset = 0.0f; }
+        else LS_TRY(ntk_rmsnorm_offset(cq_, m.q_norm, nullptr, nullptr, m.q_rank, a_, na, T, m.q_rank, eps_, 0.0f, stream_));
+        LS_TRY(ntk_dense(&d, stream_));
         q = q_;
         ldq = H * qd;
     }
@@ -401,7 +411,11 @@ int LayerStackModel::portion(int slot, const int* tokens_dev, int T, int pos0, c
             LS_TRY(ntk_dense_linear(x_, W, cat_, 2 * W, loop_in_.ptr, loop_in_.dtype, T, W, 2 * W, 0, stream_));
             x_is_x0 = false;
         }
-        LS_TRY(ntk_rmsnorm_offset(h1_, L.norm1, L.has_mlp ? h2_ : nullptr, L.has_mlp ? L.norm2 : nullptr, W, x_, W, T, W, eps_, 1.0f, stream_));
+        if (T > ntk_dense_few_rows()) {
+            LS_TRY(ntk_rmsnorm_offset(h1_, L.norm1, L.has_mlp ? h2_ : nullptr, L.has_mlp ? L.norm2 : nullptr, W, x_, W, T, W, eps_, 1.0f, stream_));
+        } else if (L.has_mlp) {   // decoding: the mixer's norm runs inside its first product (run_mixer); the feed-forward's input has three readers
+            LS_TRY(ntk_rmsnorm_offset(h2_, L.norm2, nullptr, nullptr, W, x_, W, T, W, eps_, 1.0f, stream_));
+        }
         float* cache = run.cache + (size_t)slot * opt_.max_context * L.mix.row();
         LS_TRY(run_mixer(L, cache, T, pos0));
         if (L.has_mlp) LS_TRY(run_moe(L, T));
@@ -410,9 +424,15 @@ int LayerStackModel::portion(int slot, const int* tokens_dev, int T, int pos0, c
     }
     if (n_want > 0) {
         // the wanted rows only: gather, norm, head
-        LS_TRY(ntk_embed_dense(xw_, x_is_x0 ? x0_ : x_, NTK_DT_F32, want_dev, n_want, T, W, stream_));
-        LS_TRY(ntk_rmsnorm_offset(hn_, final_norm_, nullptr, nullptr, W, xw_, W, n_want, W, eps_, 1.0f, stream_));
-        LS_TRY(ntk_dense_linear(logits_out, info_.vocab, hn_, W, head_.ptr, head_.dtype, n_want, info_.vocab, W, 0, stream_));
+        const float* xs = x_is_x0 ? x0_ : x_;
+        const float* rows = xs;                       // a single decoded token is its own gather
+        if (!(T == 1 && n_want == 1)) { LS_TRY(ntk_embed_dense(xw_, xs, NTK_DT_F32, want_dev, n_want, T, W, stream_)); rows = xw_; }
+        ntk_dense_desc d{};
+        d.Y = logits_out; d.ldy = info_.vocab; d.X = rows; d.ldx = W; d.W = head_.ptr; d.wdtype = head_.dtype; d.G = 1; d.row_div = 1; d.T = n_want;
+        d.N = info_.vocab; d.K = W;
+        if (n_want <= ntk_dense_few_rows()) { d.norm_w = final_norm_; d.norm_eps = eps_; d.norm_offset = 1.0f; }   // the output norm inside the head's launch
+        else { LS_TRY(ntk_rmsnorm_offset(hn_, final_norm_, nullptr, nullptr, W, rows, W, n_want, W, eps_, 1.0f, stream_)); d.X = hn_; }
+        LS_TRY(ntk_dense(&d, stream_));
     }
     return NTK_OK;
 }
@@ -451,10 +471,13 @@ float* LayerStackModel::forward(int slot, const int* tokens, int n, const int* w
         while (w1 < n_want && want[w1] < at + T) ++w1;
         std::vector<int> rel((size_t)std::max(w1 - done_want, 1));
         for (int i = done_want; i < w1; ++i) rel[(size_t)(i - done_want)] = want[i] - at;
-        // (blocking copies of a few integers: the previous pass has consumed the buffers once these return after a stream sync)
+        // the pinned staging area is free once the previous pass's copy has run: wait for the stream (idle already after a copy_logits), then one
+        // stream-ordered copy brings the tokens and the wanted places
         if (ntk_stream_synchronize(stream_) != NTK_OK) { err_ = "forward: the stream failed"; return nullptr; }
-        nt_hip_memcpy_h2d(tokens_dev_, tokens + at, (size_t)T * sizeof(int));
-        if (w1 > done_want) nt_hip_memcpy_h2d(want_dev_, rel.data(), (size_t)(w1 - done_want) * sizeof(int));
+        memcpy(h_stage_, tokens + at, (size_t)T * sizeof(int));
+        const int nw = w1 - done_want;
+        if (nw > 0) memcpy(h_stage_ + chunk_, rel.data(), (size_t)nw * sizeof(int));
+        if (ntk_memcpy_h2d_async(tokens_dev_, h_stage_, (size_t)(nw > 0 ? chunk_ + nw : T) * sizeof(int), stream_) != NTK_OK) { err_ = "forward: the copy of the tokens failed"; return nullptr; }
         const int st = portion(slot, tokens_dev_, T, pos0 + at, want_dev_, w1 - done_want, logits_ + (size_t)done_want * info_.vocab);
         if (st != NTK_OK) { if (err_.empty()) err_ = std::string("forward: ") + ntk_status_string(st); return nullptr; }
         done_want = w1;

@@ -122,6 +122,7 @@ private:
           *att_ = nullptr, *kx_ = nullptr, *vx_ = nullptr, *mix_ = nullptr, *wts_ = nullptr, *sg_ = nullptr, *gu_ = nullptr, *act_ = nullptr, *dn_ = nullptr,
           *sgu_ = nullptr, *sact_ = nullptr, *sdn_ = nullptr, *scratch_ = nullptr, *xw_ = nullptr, *hn_ = nullptr;
     int *ids_ = nullptr, *offsets_ = nullptr, *order_ = nullptr, *where_ = nullptr, *tokens_dev_ = nullptr, *want_dev_ = nullptr;
+    int* h_stage_ = nullptr;          // pinned: tokens and wanted places of the pass being launched
     float* logits_ = nullptr;
     size_t logits_rows_ = 0;
     int last_rows_ = 0;

@@ -115,6 +115,22 @@ def test_few_row_product_with_the_clipped_glu_inside(dtype, T, ff, K):
     assert rel(Lr.dense(x, w, dtype, glu_limit=1.5), Lr.clipped_glu(Lr.dense(x, w, dtype), 1.5)) < 1e-6
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("offset", [0.0, 1.0])
+def test_few_row_product_with_the_norm_inside(dtype, offset):
+    """decoding: the RMS norm of the activation row inside the product's launch == norm, then product"""
+    from ntransformer_amd import layers as Lr
+    g = np.random.default_rng(int(offset) + 3)
+    for T, N, K in [(1, 24, 40), (5, 70, 100), (8, 33, 264)]:
+        x = (g.standard_normal((T, K)) * 4).astype(np.float32)
+        w = O.bf16_round(torch.tensor(g.standard_normal((N, K)) / math.sqrt(K))).numpy()
+        nw = (0.2 * g.standard_normal(K) + (1.0 - offset)).astype(np.float32)
+        xt = torch.tensor(x, dtype=O.F)
+        normed = O.rms_unit(xt, 1e-5) * (offset + torch.tensor(nw, dtype=O.F))
+        got = Lr.dense(x, w, dtype, norm_w=nw, norm_eps=1e-5, norm_offset=offset)
+        assert rel(got, normed @ torch.tensor(w, dtype=O.F).T) < (1e-5 if dtype == "float32" else 1e-2)
+
+
 def test_dense_accumulates_onto_start_values():
     from ntransformer_amd import layers as Lr
     g = np.random.default_rng(9)
