@@ -384,6 +384,8 @@ def test_slots_side_by_side_freed_and_used_again(tmp_path):
     dict(layers=("latent_attention", "latent_attention_2"), mlp_on=(False, True), loop=(0, 1, 1)),           # a layer without feed-forward, one pass
     dict(layers=("latent_attention", "latent_attention_2"), width=128, heads=4, dim=32, rot_dim=16, vdim=72, kv_rank=80, q_rank=48, experts=9, top=3,
          ff=56, shared_ff=24, window=33),                                                                        # value rows and latents past one 64-column slab
+    dict(layers=("latent_attention", "latent_attention_2"), width=128, heads=3, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=96, experts=4, top=2,
+         ff=64, shared_ff=64, window=20, vocab=64),                                                              # head sizes of a full-sized model: 8 latent slabs, 2 latent columns per thread
 ])
 def test_other_sizes_and_degenerate_values(tmp_path, kw):
     cfg = O.small_config(**kw)
