@@ -315,11 +315,14 @@ __global__ __launch_bounds__(256) void dense_gemv_kernel(const DenseArgs a) {
 template <typename WT>
 static void launch_gemv(const DenseArgs& a, int rows, hipStream_t s) {
     const size_t lds = ((size_t)a.K * 4 + 15) & ~(size_t)15;
-    // outputs per workgroup 4 * RW: keep about two workgroups per CU where the matrix allows
+    // Rows per wave, measured over layer-like shapes (2048 .. 64000 outputs of 768 .. 4096 inputs, 1 .. 6 activation rows): two rows per wave are
+    // the best or within noise everywhere from 4096 outputs x rows on (a 64000 x 4096 head: 84 us against 98 with one or eight), one below; launches
+    // under ~20 MB sit at 4 - 6 us whatever the choice.  The GLU form keeps pairs: 4 pairs per wave for the large expert launches.
     const long long work = (long long)a.N * rows;
-    const int rw = work >= 4 * 8 * 512 ? 8 : work >= 4 * 4 * 512 ? 4 : work >= 4 * 2 * 512 ? 2 : 1;
+    int rw = work >= 4096 ? 2 : 1;
+    if (const int force = NTK_TUNE_ENV_INT("NTK_DENSE_GEMV_RW", 0)) rw = force;   // (tuning builds only)
     if (a.glu_ff > 0) {
-        const int out = rw >= 4 ? rw / 2 : 1;               // (gate, up) pairs per wave
+        const int out = work >= 4 * 8 * 512 ? 4 : work >= 4 * 4 * 512 ? 2 : 1;   // (gate, up) pairs per wave
         const dim3 grid((a.glu_ff + 4 * out - 1) / (4 * out), rows, 1);
         if (out == 4) hipLaunchKernelGGL((dense_gemv_kernel<WT, 8, true>), grid, dim3(256), lds, s, a);
         else if (out == 2) hipLaunchKernelGGL((dense_gemv_kernel<WT, 4, true>), grid, dim3(256), lds, s, a);
