@@ -37,8 +37,8 @@ int main(int argc, char** argv) {
     if (dtype != "bfloat16" && dtype != "float32") { fprintf(stderr, "--dtype must be bfloat16 or float32\n"); return 2; }
     if (max_tokens < 1) max_tokens = 1;
     nt::SeqLoadOptions opt;
-    opt.max_context = max_tokens;   // one request at a time may hold all of them
-    opt.slots = 1;
+    opt.max_context = max_tokens;   // one request may hold all of them
+    opt.slots = 4;                  // requests normally come one after the other; a few may overlap
     opt.float32 = dtype == "float32";
     std::string why;
     std::unique_ptr<nt::SequenceModel> m = nt::open_model(model, opt, &why);

@@ -449,18 +449,24 @@ def test_trace_runner_replays_steps(tmp_path):
         {"step": 1, "entries": [{"id": "a", "tokens": ta[13:15], "want": []}], "end": []},
         {"step": 2, "entries": [{"id": "a", "tokens": ta[15:], "want": [4]}], "end": ["a"]},
         {"step": 3, "entries": [{"id": "b", "tokens": tb, "want": [5]}], "end": ["b"]},
+        # two requests alive at once, portions alternating
+        {"step": 4, "entries": [{"id": "c", "tokens": ta[:9], "want": []}], "end": []},
+        {"step": 5, "entries": [{"id": "d", "tokens": tb[:2], "want": [1]}], "end": []},
+        {"step": 6, "entries": [{"id": "c", "tokens": ta[9:], "want": [10]}, {"id": "d", "tokens": tb[2:], "want": [3]}], "end": ["c", "d"]},
     ]
     out = tmp_path / "out"
     out.mkdir()
     r = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--out", str(out), "--max-tokens", "20"],
                        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stderr[-2000:]
-    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2", "done 3"]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done %d" % k for k in range(7)]
     assert not (out / "1.f32").exists()
     V = cfg["vocab"]
     assert rel(np.fromfile(out / "0.f32", np.float32).reshape(-1, V), ra[[0, 12]]) < TOL["float32"]
     assert rel(np.fromfile(out / "2.f32", np.float32).reshape(-1, V), ra[[19]]) < TOL["float32"]
     assert rel(np.fromfile(out / "3.f32", np.float32).reshape(-1, V), rb[[5]]) < TOL["float32"]
+    assert rel(np.fromfile(out / "5.f32", np.float32).reshape(-1, V), rb[[1]]) < TOL["float32"]
+    assert rel(np.fromfile(out / "6.f32", np.float32).reshape(-1, V), np.stack([ra[19], rb[5]])) < TOL["float32"]
 
 
 def test_a_folder_with_an_unknown_architecture_or_a_missing_tensor_is_refused(tmp_path):
