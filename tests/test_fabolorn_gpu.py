@@ -386,6 +386,8 @@ def test_slots_side_by_side_freed_and_used_again(tmp_path):
          ff=56, shared_ff=24, window=33),                                                                        # value rows and latents past one 64-column slab
     dict(layers=("latent_attention", "latent_attention_2"), width=128, heads=3, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=96, experts=4, top=2,
          ff=64, shared_ff=64, window=20, vocab=64),                                                              # head sizes of a full-sized model: 8 latent slabs, 2 latent columns per thread
+    dict(layers=("latent_attention_2", "latent_attention"), experts=130, top=9, ff=8, shared_ff=0, window=1000, heads=5, loop=(0, 2, 3)),   # many experts (three per lane),
+                                                                                                                 # more picks than few-row products take, a window wider than the sequence
 ])
 def test_other_sizes_and_degenerate_values(tmp_path, kw):
     cfg = O.small_config(**kw)
