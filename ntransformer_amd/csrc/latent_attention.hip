@@ -375,7 +375,15 @@ __global__ __launch_bounds__(256) void latent_attention_merge_kernel(float* out,
     float* o = out + (long long)(r / H) * ldo + (long long)(r % H) * nV;
     for (int v = threadIdx.x; v < nV; v += 256) {
         float s2 = 0.0f;
-        for (int s = 0; s < splits; ++s) s2 = fmaf(st[(long long)s * (2 + nV) + 2 + v], wt[s], s2);
+        int s = 0;
+        for (; s + 8 <= splits; s += 8) {          // eight states requested together, added in order
+            float x[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) x[u] = st[(long long)(s + u) * (2 + nV) + 2 + v];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s2 = fmaf(x[u], wt[s + u], s2);
+        }
+        for (; s < splits; ++s) s2 = fmaf(st[(long long)s * (2 + nV) + 2 + v], wt[s], s2);
         o[v] = s2 * inv;
     }
 }
