@@ -35,11 +35,14 @@ typedef struct ntk_dense_desc {
     int T, N, K;
     int accumulate;
     /* glu_ff > 0 (only with T <= ntk_dense_few_rows(), N == 2 * glu_ff, no accumulate): W holds glu_ff gate rows then glu_ff up rows and
-     * Y[r][f] = g' * sigmoid(glu_alpha * g') * (u' + 1), g' = min(gate, glu_limit), u' = clamp(up, -glu_limit, glu_limit) -- the product and ntk_clipped_glu in one launch */
+     * Y[r][f] = g' * sigmoid(glu_alpha * g') * (u' + glu_up_offset), g' = min(gate, glu_limit), u' = clamp(up, -glu_limit, glu_limit) -- the product and ntk_clipped_glu in one launch */
     int glu_ff; float glu_limit, glu_alpha;
     /* norm_w != NULL (only with T <= ntk_dense_few_rows()): every activation row is first divided by sqrt(mean(x^2) + norm_eps) and multiplied by
      * (norm_offset + norm_w[k]), norm_w F32 [K] -- ntk_rmsnorm_offset and the product in one launch */
     const float* norm_w; float norm_eps, norm_offset;
+    /* what is added to the (clamped) up value inside the gated activation: 1 for the clipped form above, 0 for a plain gated unit
+     * (g * sigmoid(alpha * g) * u; glu_limit = INFINITY switches the clamps off: silu(g) * u with alpha 1) */
+    float glu_up_offset;
 } ntk_dense_desc;
 int ntk_dense_few_rows(void);   /* up to this many rows a product takes the row-streaming form */
 int ntk_dense(const ntk_dense_desc* d, void* stream);
@@ -61,6 +64,27 @@ int ntk_sigmoid_gate(float* y, int ldy, const float* g, int ldg, int T, int n, v
 int ntk_rows_copy(float* dst, const float* src, long long n, void* stream);
 /* x[i] += a[i] (+ b[i] if b) */
 int ntk_residual_add(float* x, const float* a, const float* b, int n, void* stream);
+
+/* out[t][:] = table[tokens[t]][:] * scale */
+int ntk_embed_dense_scaled(float* out, const void* table, int tdtype, const int* tokens, int T, int vocab, int width, float scale, void* stream);
+/* x[i] *= s */
+int ntk_scale(float* x, long long n, float s, void* stream);
+/* Layer norm with weight and bias: y[t][:] (+)= (x[t] - mean) / sqrt(var + eps) * w + b, var = mean of the squared deviations (two passes).
+ * b may be NULL (no bias); accumulate != 0 adds onto y (the residual sum of a layer whose sublayer output is normed before it is added). */
+int ntk_layernorm(float* y, int ldy, const float* x, int ldx, const float* w, const float* b, int T, int n, float eps, int accumulate, void* stream);
+/* The input side of a causal convolution over time that is ADDED to its input (out = h + conv(h)), h = layer norm of x:
+ * ntk_layernorm_history fills hist [(taps - 1) + T][n]: rows 0 .. taps-2 = the last taps-1 inputs h of the sequence before this portion (from
+ * `state` [taps - 1][n]; zeros where the position lies before the sequence's start, i.e. pos0 - (taps-1) + k < 0), rows taps-1 .. = layer norm of x[t].
+ * ntk_causal_conv_mix then gives out[t][c] = hist[taps-1+t][c] + sum_j w[c][j] * hist[t+j][c] (w F32 [n][taps], tap taps-1 is the present token)
+ * and leaves the portion's last taps-1 rows of hist in `state` for the next portion.  taps >= 1 (taps 1: no state is read or written). */
+int ntk_layernorm_history(float* hist, const float* x, int ldx, const float* w, const float* b, const float* state, int taps, int pos0, int T, int n, float eps,
+                          void* stream);
+int ntk_causal_conv_mix(float* out, int ldo, const float* hist, const float* w, float* state, int taps, int T, int n, void* stream);
+/* y[t][i] = a N(z)_i + b N(z^2)_i + c N(z^3)_i + e with (a, b, c, e) = coef[0..3] (device F32), powers element by element and
+ * N(u) = u / sqrt(mean(u^2) + eps) over the row of n values */
+int ntk_polynorm(float* y, int ldy, const float* z, int ldz, const float* coef, int T, int n, float eps, void* stream);
+/* y[t][i] = x[t][i] / sqrt(mean(x[t]^2) + eps) * w[i] * sigmoid(g[t][i]) (the norm runs over the whole row of n values; g rows ldg apart, g may be NULL) */
+int ntk_gated_rmsnorm(float* y, int ldy, const float* x, int ldx, const float* w, const float* g, int ldg, int T, int n, float eps, void* stream);
 
 /* ---- latent_attention.hip ---------------------------------------------------------------------------------------------------------
  * Attention whose keys and values are up-projections of one cached latent per position plus one rotated key part shared by the heads.
@@ -93,16 +117,65 @@ int ntk_latent_fold_query(float* qf, const float* q, int ldq, const void* w_uk, 
 int ntk_latent_unfold_value(float* out, int ldo, const float* lat, const void* w_uv, int wdtype, const float* gate, int ldg, int T, int H, int dv, int R,
                             void* stream);
 
+/* ---- window_attention.hip ---------------------------------------------------------------------------------------------------------
+ * Grouped-query softmax attention over a cache of rotated keys and values, causal with an optional sliding window, with `maps` (1 or 2) score maps per
+ * head that share the values.  Cache row of a position: [G][maps][dn] rotated keys | [G][dv] values (row >= G * (maps * dn + dv) floats).
+ * Query head h uses key/value head h / (H / G); q [T][H][maps][dn].
+ * ntk_window_prepare rotates q in place and k into the cache rows pos0 .. pos0+T-1 (the first rot->dims entries of every map of every head, neighbours
+ * (2i, 2i+1) paired; the rest unchanged) and copies v behind the keys. */
+int ntk_window_prepare(float* cache, int row, float* q, int ldq, const float* k, int ldk, const float* v, int ldv, int H, int G, int maps, int dn, int dv,
+                       const ntk_rotary* rot, int pos0, int T, void* stream);
+/* a_m = softmax_j(scale * q_m . k_m[j]) V over the visible j (j <= p, and p - j < window if window > 0), per map m.
+ * maps == 1: out = a_0.  maps == 2: out = a_0 - lambda * a_1 (a differential pair).  sub_norm != 0: out is then divided by sqrt(mean(out^2) + eps) over
+ * the head's dv values.  out_scale multiplies the result.  out [T][H][dv], ldo floats between tokens.
+ * Long key ranges of few query rows are cut into `splits` parts that a second launch merges: scratch F32 [>= ntk_window_attention_scratch(...)] (may be NULL when that is 0). */
+typedef struct ntk_window_attention_desc {
+    float* out; int ldo;
+    const float* q; int ldq;
+    const float* cache; int row;
+    int H, G, maps, dn, dv;
+    int pos0, T, window;
+    float scale, lambda;
+    int sub_norm; float eps, out_scale;
+    float* scratch;
+} ntk_window_attention_desc;
+size_t ntk_window_attention_scratch(int T, int H, int maps, int dv, int nkeys);
+int ntk_window_attention(const ntk_window_attention_desc* d, void* stream);
+
+/* ---- lightning_attention.hip -------------------------------------------------------------------------------------------------------
+ * Linear attention with a per-head decay: S_t = decay_h S_(t-1) + k_t v_t^T (S [dn][dv] per head, F32), o_t = S_t^T q_t, with q, k, v = act(raw)
+ * (act = silu when silu != 0) applied on the way in.  Portions are walked in chunks (scores inside a chunk, the state between chunks), all in F32.
+ * q [T][H][dn], k [T][H][dn], v [T][H][dv] with ldq / ldk / ldv floats between tokens; log_decay device F32 [H] = ln(decay_h) (-inf for 0);
+ * state [H][dn][dv]: read unless pos0 == 0 (a sequence starts from zeros), written at the end.  out [T][H][dv].  dn <= 256. */
+int ntk_lightning_attention(float* out, int ldo, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* log_decay, float* state,
+                            int H, int dn, int dv, int silu, int pos0, int T, void* stream);
+
 /* ---- moe.hip ---------------------------------------------------------------------------------------------------------------------- */
 /* Router of a mixture of experts, one launch: z = W_r h (F32 weights [E][n]), s = softmax(z); the `top` largest (ties: the lower index), weights
  * s / (sum of the chosen + 1e-20) -> ids [T][top], wts [T][top].  shared_gate_w (F32 [n], may be NULL) -> sgate[t] = sigmoid(w . h[t]).  E <= 256. */
 int ntk_moe_route(int* ids, float* wts, float* sgate, const float* h, int ldh, const float* w_router, const float* shared_gate_w, int T, int n, int E, int top,
                   void* stream);
+/* The general router.  score 0: s = softmax(z), 1: s = sigmoid(z).  groups > 1: the experts form `groups` equal groups of neighbours, a group's
+ * score is the sum of its `group_top` largest s, and only experts of the `keep` best groups can be chosen (ties: the lower index).  The `top` largest
+ * allowed s are chosen; weights = s (renorm != 0: divided by the sum of the chosen + 1e-20) * scale. */
+typedef struct ntk_route_desc {
+    int score;
+    int groups, keep, group_top;
+    int renorm;
+    float scale;
+} ntk_route_desc;
+int ntk_moe_route_ex(int* ids, float* wts, float* sgate, const float* h, int ldh, const float* w_router, const float* shared_gate_w, int T, int n, int E, int top,
+                     const ntk_route_desc* r, void* stream);
 /* Stable grouping of the T*top (token, slot) pairs by expert: offsets [E+1], order [T*top] (pair index t*top+slot of every sorted row),
  * where [T*top] (sorted row of every pair). */
 int ntk_moe_group(int* offsets, int* order, int* where, const int* ids, int T, int top, int E, void* stream);
 /* a[r][f] = g' * sigmoid(alpha * g') * (u' + 1), g' = min(gu[r][f], limit), u' = clamp(gu[r][ff + f], -limit, limit); gu rows of 2*ff, a rows of ff */
 int ntk_clipped_glu(float* a, const float* gu, int rows, int ff, float limit, float alpha, void* stream);
+/* the general gated unit: a[r][f] = g' * sigmoid(alpha * g') * (u' + up_offset) with the clamps of ntk_clipped_glu (limit = INFINITY: none) */
+int ntk_glu(float* a, const float* gu, int rows, int ff, float limit, float alpha, float up_offset, void* stream);
+/* out[t][:] = sum_s wts[t][s] * d[where[t*top+s]][:] + (sgate ? sgate[t] : 1) * shared[t][:] (if shared): the experts' sum on its own, for layers that norm it before
+ * it joins the stream */
+int ntk_moe_sum(float* out, const float* d, const int* where, const float* wts, const float* shared, const float* sgate, int T, int top, int n, void* stream);
 /* x[t][:] += mix[t][:] (if mix) + sum_s wts[t][s] * d[where[t*top+s]][:] + sgate[t] * shared[t][:] (if shared) -- slots in order, one rounding sequence per token */
 int ntk_moe_combine(float* x, const float* mix, const float* d, const int* where, const float* wts, const float* shared, const float* sgate, int T, int top,
                     int n, void* stream);

@@ -13,8 +13,15 @@ namespace nt {
         if (st__ != NTK_OK) return st__;      \
     } while (0)
 
-static constexpr float kGluAlpha = 1.702f;   // the design fixes the slope of the experts' gate activation
-static FamilyRegistrar reg_fabolorn("Fabolorn", [] { return std::unique_ptr<SequenceModel>(new LayerStackModel()); });
+static constexpr float kGluAlpha = 1.702f;   // the slope of the clipped gated unit's activation
+static StackForm parallel_form() { return StackForm{}; }
+static StackForm sequential_form() {
+    StackForm f;
+    f.sequential = true; f.loop_projection = false; f.router_score = 1; f.router_renorm = false; f.clipped_glu = false; f.shared_gate = false; f.group_top = 2;
+    return f;
+}
+static FamilyRegistrar reg_fabolorn("Fabolorn", [] { return std::unique_ptr<SequenceModel>(new LayerStackModel(parallel_form())); });
+static FamilyRegistrar reg_nizorax("Nizorax", [] { return std::unique_ptr<SequenceModel>(new LayerStackModel(sequential_form())); });
 
 LayerStackModel::~LayerStackModel() {
     if (stream_) ntk_stream_synchronize(stream_);
@@ -84,11 +91,121 @@ int LayerStackModel::parse_mixer(const Json& L, const std::string& type, LatentM
     return NTK_OK;
 }
 
+// rotary frequencies base^(-2i/dims), optionally rescaled by wavelength: kept below original/high, divided by factor above original/low, blended between
+static std::vector<double> wavelength_scaled_frequencies(const Json& rot, int dims) {
+    const double base = rot.at("base").number(10000.0);
+    const int half = dims / 2;
+    std::vector<double> f((size_t)std::max(half, 1));
+    for (int i = 0; i < half; ++i) f[(size_t)i] = std::pow(base, -2.0 * i / dims);
+    if (rot.has("scaling")) {
+        const Json& sc = rot.at("scaling");
+        const double factor = sc.at("factor").number(1.0), orig = sc.at("original").number(1.0), low = sc.at("low").number(1.0), high = sc.at("high").number(1.0);
+        for (int i = 0; i < half; ++i) {
+            const double fr = f[(size_t)i], wl = 2.0 * M_PI / fr;
+            if (wl < orig / high) continue;
+            if (wl > orig / low) { f[(size_t)i] = fr / factor; continue; }
+            const double sm = (orig / wl - low) / (high - low);
+            f[(size_t)i] = (1.0 - sm) * fr / factor + sm * fr;
+        }
+    }
+    return f;
+}
+
+int LayerStackModel::parse_window(const Json& L, WindowMixer& m) {
+    const Json& mx = L.at("mixer");
+    const std::string where = "mixer 'attention'";
+    if (!mx.is_object()) return fail(NTK_E_FORMAT, where + ": no 'mixer' object");
+    if (!need_int(mx, "heads", m.heads, err_, where) || !need_int(mx, "dim", m.dim, err_, where) || !need_int(mx, "vdim", m.vdim, err_, where)) return NTK_E_FORMAT;
+    m.kv_heads = m.heads;
+    if (mx.has("kv_heads") && !need_int(mx, "kv_heads", m.kv_heads, err_, where)) return NTK_E_FORMAT;
+    if (m.heads % m.kv_heads) return fail(NTK_E_FORMAT, where + ": heads must be a multiple of kv_heads");
+    if (!mx.at("scale").is_number()) return fail(NTK_E_FORMAT, where + ": 'scale' is missing");
+    m.scale = (float)mx.at("scale").number();
+    m.maps = mx.has("diff") ? 2 : 1;
+    m.diff = (float)mx.at("diff").number(0.0);
+    m.window = 0;
+    if (mx.has("mask") && !need_int(mx.at("mask"), "size", m.window, err_, where + " mask")) return NTK_E_FORMAT;
+    m.rot_dims = 0;
+    std::vector<double> f(1, 0.0);
+    if (mx.has("rot")) {
+        const Json& rot = mx.at("rot");
+        m.rot_dims = rot.has("dims") ? (int)rot.at("dims").integer() : m.dim;
+        if (m.rot_dims < 0 || (m.rot_dims & 1) || m.rot_dims > m.dim) return fail(NTK_E_FORMAT, where + ": rot.dims must be even and at most dim");
+        f = wavelength_scaled_frequencies(rot, m.rot_dims);
+    }
+    m.rot_freq = (double*)dev_alloc(f.size() * sizeof(double));
+    if (!m.rot_freq) return fail(NTK_E_NOMEM, "out of device memory");
+    nt_hip_memcpy_h2d(m.rot_freq, f.data(), f.size() * sizeof(double));
+    return NTK_OK;
+}
+
+int LayerStackModel::parse_lightning(const Json& L, LightningMixer& m) {
+    const Json& mx = L.at("mixer");
+    const std::string where = "mixer 'lightning'";
+    if (!mx.is_object()) return fail(NTK_E_FORMAT, where + ": no 'mixer' object");
+    if (!need_int(mx, "heads", m.heads, err_, where) || !need_int(mx, "dim", m.dim, err_, where) || !need_int(mx, "vdim", m.vdim, err_, where)) return NTK_E_FORMAT;
+    if (m.dim > 256) return fail(NTK_E_SHAPE, where + ": dim up to 256 is supported");
+    const Json& dc = mx.at("decay");
+    std::vector<float> ld((size_t)m.heads);
+    for (int h = 0; h < m.heads; ++h) {
+        double d;
+        if (dc.is_number()) d = dc.number();
+        else if (dc.is_array() && (int)dc.arr.size() == m.heads && dc.arr[(size_t)h].is_number()) d = dc.arr[(size_t)h].number();
+        else return fail(NTK_E_FORMAT, where + ": 'decay' must be a number or one number per head");
+        if (d < 0.0 || d > 1.0) return fail(NTK_E_FORMAT, where + ": a decay lies in [0, 1]");
+        ld[(size_t)h] = d > 0.0 ? (float)std::log(d) : -INFINITY;
+    }
+    m.log_decay = (float*)dev_alloc(ld.size() * sizeof(float));
+    if (!m.log_decay) return fail(NTK_E_NOMEM, "out of device memory");
+    nt_hip_memcpy_h2d(m.log_decay, ld.data(), ld.size() * sizeof(float));
+    return NTK_OK;
+}
+
+int LayerStackModel::parse_mlp(const Json& ml, const std::string& where, StackLayer& S) {
+    const std::string kind = ml.at("kind").is_string() ? ml.at("kind").str : "moe";
+    if (kind == "dense") {
+        S.mlp_kind = kMlpDense;
+        if (!need_int(ml, "ff", S.ffn.ff, err_, where)) return NTK_E_FORMAT;
+        return NTK_OK;
+    }
+    if (kind != "moe") return fail(NTK_E_FORMAT, where + ": unknown kind '" + kind + "'");
+    S.mlp_kind = kMlpMoe;
+    MoeFeedForward& M = S.mlp;
+    const Json& rt = ml.at("router");
+    if (!need_int(rt, "experts", M.experts, err_, where) || !need_int(rt, "top", M.top, err_, where) || !need_int(ml.at("expert"), "ff", M.routed.ff, err_, where))
+        return NTK_E_FORMAT;
+    if (M.top > M.experts || M.experts > 255) return fail(NTK_E_FORMAT, where + ": top <= experts <= 255 is required");
+    M.route.score = form_.router_score;
+    M.route.renorm = form_.router_renorm ? 1 : 0;
+    M.route.scale = (float)rt.at("scale").number(1.0);
+    M.route.groups = 1; M.route.keep = 1; M.route.group_top = form_.group_top;
+    if (rt.has("groups")) {
+        if (!need_int(rt.at("groups"), "count", M.route.groups, err_, where + " groups") || !need_int(rt.at("groups"), "keep", M.route.keep, err_, where + " groups")) return NTK_E_FORMAT;
+        if (M.experts % M.route.groups || M.route.keep > M.route.groups || (long long)M.route.keep * (M.experts / M.route.groups) < M.top)
+            return fail(NTK_E_FORMAT, where + ": groups must divide the experts and the kept groups must hold 'top' experts");
+    }
+    if (form_.clipped_glu) { M.glu_alpha = kGluAlpha; M.glu_up_offset = 1.0f; M.routed.limit = (float)ml.at("expert").at("limit").number(); }
+    else { M.glu_alpha = 1.0f; M.glu_up_offset = 0.0f; M.routed.limit = INFINITY; }
+    M.has_shared = ml.has("shared");
+    if (M.has_shared) {
+        if (!need_int(ml.at("shared"), "ff", M.shared.ff, err_, where + " shared")) return NTK_E_FORMAT;
+        M.shared.limit = form_.clipped_glu ? (float)ml.at("shared").at("limit").number() : INFINITY;
+    }
+    return NTK_OK;
+}
+
 int LayerStackModel::parse(const ModelFolder& f) {
     const Json& c = f.config();
     info_.architecture = c.at("architecture").str;
     if (!need_int(c, "vocab", info_.vocab, err_, "config") || !need_int(c, "width", info_.width, err_, "config")) return NTK_E_FORMAT;
     eps_ = (float)c.at("norm").at("eps").number(1e-6);
+    if (form_.sequential) {
+        taps_ = (int)c.at("canon").at("taps").integer(1);
+        if (taps_ < 1 || taps_ > 64) return fail(NTK_E_FORMAT, "config: canon.taps must lie in 1 .. 64");
+        embed_scale_ = (float)c.at("embedding").at("scale").number(1.0);
+        logit_scale_ = (float)c.at("logit_scale").number(1.0);
+        has_state_ = taps_ > 1;
+    }
     if (c.at("bos").is_number()) info_.bos = (int)c.at("bos").integer();
     if (c.at("eos").is_number()) info_.eos = (int)c.at("eos").integer();
     const Json& ls = c.at("layers");
@@ -98,25 +215,14 @@ int LayerStackModel::parse(const ModelFolder& f) {
         const Json& L = ls.arr[i];
         StackLayer& S = layers_[i];
         S.type = L.at("type").str;
-        if (S.type != "latent_attention" && S.type != "latent_attention_2") return fail(NTK_E_FORMAT, "layer " + std::to_string(i) + ": unknown mixer type '" + S.type + "'");
-        LS_TRY(parse_mixer(L, S.type, S.mix));
+        // which mixers a form lists: the parallel form's layers read two norms of one input, so its mixers are the latent kinds it was built around
+        if (!form_.sequential && (S.type == "latent_attention" || S.type == "latent_attention_2")) { S.mixer = kMixLatent; LS_TRY(parse_mixer(L, S.type, S.mix)); }
+        else if (form_.sequential && S.type == "attention") { S.mixer = kMixWindow; LS_TRY(parse_window(L, S.att)); }
+        else if (form_.sequential && S.type == "lightning") { S.mixer = kMixLightning; LS_TRY(parse_lightning(L, S.lin)); has_state_ = true; }
+        else return fail(NTK_E_FORMAT, "layer " + std::to_string(i) + ": unknown mixer type '" + S.type + "'");
         S.has_mlp = L.has("mlp");
-        if (S.has_mlp) {
-            const Json& ml = L.at("mlp");
-            const std::string where = "layer " + std::to_string(i) + " mlp";
-            if (ml.at("kind").is_string() && ml.at("kind").str != "moe") return fail(NTK_E_FORMAT, where + ": unknown kind '" + ml.at("kind").str + "'");
-            MoeFeedForward& M = S.mlp;
-            if (!need_int(ml.at("router"), "experts", M.experts, err_, where) || !need_int(ml.at("router"), "top", M.top, err_, where) ||
-                !need_int(ml.at("expert"), "ff", M.routed.ff, err_, where))
-                return NTK_E_FORMAT;
-            if (M.top > M.experts || M.experts > 255) return fail(NTK_E_FORMAT, where + ": top <= experts <= 255 is required");
-            M.routed.limit = (float)ml.at("expert").at("limit").number();
-            M.has_shared = ml.has("shared");
-            if (M.has_shared) {
-                if (!need_int(ml.at("shared"), "ff", M.shared.ff, err_, where + " shared")) return NTK_E_FORMAT;
-                M.shared.limit = (float)ml.at("shared").at("limit").number();
-            }
-        }
+        if (S.has_mlp) LS_TRY(parse_mlp(L.at("mlp"), "layer " + std::to_string(i) + " mlp", S));
+        if (!form_.sequential && S.mlp_kind == kMlpDense) return fail(NTK_E_FORMAT, "layer " + std::to_string(i) + ": this family has no dense feed-forward");
     }
     // the order of layer runs
     const int n = (int)layers_.size();
@@ -126,12 +232,12 @@ int LayerStackModel::parse(const ModelFolder& f) {
         const Json& lp = c.at("loop");
         const int a = (int)lp.at("start").integer(), b = (int)lp.at("stop").integer(), times = (int)lp.at("times").integer(1);
         if (a < 0 || b <= a || b > n || times < 1) return fail(NTK_E_FORMAT, "config: loop needs 0 <= start < stop <= layers and times >= 1");
-        for (int i = 0; i < a; ++i) runs_.push_back({i, false, nullptr});
+        for (int i = 0; i < a; ++i) runs_.push_back({i, false, nullptr, nullptr, nullptr});
         for (int t = 0; t < times; ++t)
-            for (int i = a; i < b; ++i) runs_.push_back({i, i == a, nullptr});
-        for (int i = b; i < n; ++i) runs_.push_back({i, false, nullptr});
+            for (int i = a; i < b; ++i) runs_.push_back({i, form_.loop_projection && i == a, nullptr, nullptr, nullptr});
+        for (int i = b; i < n; ++i) runs_.push_back({i, false, nullptr, nullptr, nullptr});
     } else {
-        for (int i = 0; i < n; ++i) runs_.push_back({i, false, nullptr});
+        for (int i = 0; i < n; ++i) runs_.push_back({i, false, nullptr, nullptr, nullptr});
     }
     info_.n_layers = n;
     info_.n_layer_runs = (int)runs_.size();
@@ -203,18 +309,66 @@ int LayerStackModel::upload_matrix(const ModelFolder& f, const std::vector<std::
     return NTK_OK;
 }
 
-int LayerStackModel::upload_layer(const ModelFolder& f, int i, StackLayer& L) {
-    const std::string p = "l" + std::to_string(i) + ".";
+int LayerStackModel::upload_norm(const ModelFolder& f, const std::string& name, NormW& out) {
+    LS_TRY(upload_vector(f, name, info_.width, &out.w));
+    if (form_.sequential) LS_TRY(upload_vector(f, name + ".b", info_.width, &out.b));
+    return NTK_OK;
+}
+
+int LayerStackModel::upload_mixer(const ModelFolder& f, const std::string& p, int i, StackLayer& L) {
     const int W = info_.width;
+    const std::string li = "layer " + std::to_string(i);
+    if (L.mixer == kMixWindow) {
+        WindowMixer& m = L.att;
+        LS_TRY(upload_matrix(f, {p + "mix.q", p + "mix.k", p + "mix.v"}, W, m.in));
+        m.k_off = m.heads * m.maps * m.dim;
+        m.v_off = m.k_off + m.kv_heads * m.maps * m.dim;
+        if (m.in.out_f != m.v_off + m.kv_heads * m.vdim) return fail(NTK_E_SHAPE, li + ": the mixer's input projections do not have the configured sizes");
+        const StTensor* tq = f.tensor(p + "mix.q");
+        if (!tq || tq->shape[0] != m.k_off) return fail(NTK_E_SHAPE, "tensor '" + p + "mix.q' does not have heads * maps * dim rows");
+        LS_TRY(upload_matrix(f, {p + "mix.o"}, (int64_t)m.heads * m.vdim, m.o));
+        if (m.o.out_f != W) return fail(NTK_E_SHAPE, "tensor '" + p + "mix.o' does not have 'width' rows");
+        m.lambda = 0.0f;
+        if (m.maps == 2) {
+            // lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff, one number for the layer, in F32
+            float dots[2];
+            for (int k = 0; k < 2; ++k) {
+                const StTensor* a = f.tensor(p + "mix.lq" + std::to_string(k + 1));
+                const StTensor* b = f.tensor(p + "mix.lk" + std::to_string(k + 1));
+                if (!a || !b) return fail(NTK_E_FORMAT, "tensor '" + p + "mix.lq" + std::to_string(k + 1) + "' or its 'lk' is missing");
+                if (a->numel() != m.dim || b->numel() != m.dim) return fail(NTK_E_SHAPE, li + ": the lambda vectors must have 'dim' entries");
+                std::vector<float> va((size_t)m.dim), vb((size_t)m.dim);
+                if (!tensor_to_f32(*a, va.data()) || !tensor_to_f32(*b, vb.data())) return fail(NTK_E_DTYPE, li + ": lambda vectors of an unsupported dtype");
+                float sdot = 0.0f;
+                for (int d = 0; d < m.dim; ++d) sdot = std::fma(va[(size_t)d], vb[(size_t)d], sdot);
+                dots[k] = sdot;
+                weight_bytes_ += a->nbytes + b->nbytes;
+            }
+            m.lambda = std::exp(dots[0]) - std::exp(dots[1]) + m.diff;
+        }
+        return NTK_OK;
+    }
+    if (L.mixer == kMixLightning) {
+        LightningMixer& m = L.lin;
+        const int hq = m.heads * m.dim, hv = m.heads * m.vdim;
+        LS_TRY(upload_matrix(f, {p + "mix.q", p + "mix.k", p + "mix.v", p + "mix.g"}, W, m.in));
+        m.k_off = hq; m.v_off = 2 * hq; m.g_off = 2 * hq + hv;
+        const StTensor* tq = f.tensor(p + "mix.q");
+        const StTensor* tk = f.tensor(p + "mix.k");
+        if (m.in.out_f != m.g_off + hv || !tq || !tk || tq->shape[0] != hq || tk->shape[0] != hq) return fail(NTK_E_SHAPE, li + ": the mixer's input projections do not have the configured sizes");
+        LS_TRY(upload_vector(f, p + "mix.norm", hv, &m.norm));
+        LS_TRY(upload_matrix(f, {p + "mix.o"}, hv, m.o));
+        if (m.o.out_f != W) return fail(NTK_E_SHAPE, "tensor '" + p + "mix.o' does not have 'width' rows");
+        return NTK_OK;
+    }
     LatentMixer& m = L.mix;
-    LS_TRY(upload_vector(f, p + "norm1", W, &L.norm1));
     const int hq = m.heads * m.qd(), hv = m.heads * m.vdim;
     const std::string first = m.q_rank ? p + "mix.dq" : p + "mix.q";
     LS_TRY(upload_matrix(f, {first, p + "mix.dkv", p + "mix.g"}, W, m.in));
     m.q_off = 0;
     m.kv_off = m.q_rank ? m.q_rank : hq;
     m.g_off = m.kv_off + m.row();
-    if (m.in.out_f != m.g_off + hv) return fail(NTK_E_SHAPE, "layer " + std::to_string(i) + ": the mixer's input projections do not have the configured sizes");
+    if (m.in.out_f != m.g_off + hv) return fail(NTK_E_SHAPE, li + ": the mixer's input projections do not have the configured sizes");
     if (m.q_rank) {
         LS_TRY(upload_vector(f, p + "mix.dq.norm", m.q_rank, &m.q_norm));
         LS_TRY(upload_matrix(f, {p + "mix.uq"}, m.q_rank, m.uq));
@@ -224,25 +378,55 @@ int LayerStackModel::upload_layer(const ModelFolder& f, int i, StackLayer& L) {
     LS_TRY(upload_matrix(f, {p + "mix.uk"}, m.kv_rank, m.uk));
     LS_TRY(upload_matrix(f, {p + "mix.uv"}, m.kv_rank, m.uv));
     LS_TRY(upload_matrix(f, {p + "mix.o"}, hv, m.o));
-    if (m.uk.out_f != m.heads * m.dim || m.uv.out_f != hv || m.o.out_f != W) return fail(NTK_E_SHAPE, "layer " + std::to_string(i) + ": up-projections do not have the configured sizes");
+    if (m.uk.out_f != m.heads * m.dim || m.uv.out_f != hv || m.o.out_f != W) return fail(NTK_E_SHAPE, li + ": up-projections do not have the configured sizes");
+    return NTK_OK;
+}
+
+int LayerStackModel::upload_mlp(const ModelFolder& f, const std::string& p, int i, StackLayer& L) {
+    const int W = info_.width;
+    const std::string li = "layer " + std::to_string(i);
+    if (L.mlp_kind == kMlpDense) {
+        DenseFeedForward& D = L.ffn;
+        LS_TRY(upload_matrix(f, {p + "mlp.up"}, W, D.up));
+        LS_TRY(upload_matrix(f, {p + "mlp.down"}, D.ff, D.down));
+        if (D.up.out_f != D.ff || D.down.out_f != W) return fail(NTK_E_SHAPE, li + ": feed-forward matrices do not have the configured sizes");
+        return upload_vector(f, p + "mlp.act", 4, &D.act);
+    }
+    MoeFeedForward& M = L.mlp;
+    LS_TRY(upload_vector(f, p + "mlp.router", (int64_t)M.experts * W, &M.router));
+    std::vector<std::string> gu, dn;
+    for (int e = 0; e < M.experts; ++e) {
+        const std::string q = p + "mlp.e" + std::to_string(e) + ".";
+        gu.push_back(q + "gate"); gu.push_back(q + "up"); dn.push_back(q + "down");
+    }
+    LS_TRY(upload_matrix(f, gu, W, M.routed.gate_up, M.experts));
+    LS_TRY(upload_matrix(f, dn, M.routed.ff, M.routed.down, M.experts));
+    if (M.routed.gate_up.out_f != 2 * M.routed.ff || M.routed.down.out_f != W) return fail(NTK_E_SHAPE, li + ": expert matrices do not have the configured sizes");
+    if (M.has_shared) {
+        LS_TRY(upload_matrix(f, {p + "mlp.shared.gate", p + "mlp.shared.up"}, W, M.shared.gate_up));
+        LS_TRY(upload_matrix(f, {p + "mlp.shared.down"}, M.shared.ff, M.shared.down));
+        if (M.shared.gate_up.out_f != 2 * M.shared.ff || M.shared.down.out_f != W) return fail(NTK_E_SHAPE, li + ": shared expert matrices do not have the configured sizes");
+        if (form_.shared_gate) LS_TRY(upload_vector(f, p + "mlp.shared.sg", W, &M.shared_gate));
+    }
+    return NTK_OK;
+}
+
+int LayerStackModel::upload_layer(const ModelFolder& f, int i, StackLayer& L) {
+    const std::string p = "l" + std::to_string(i) + ".";
+    const int W = info_.width;
+    LS_TRY(upload_norm(f, p + "norm1", L.norm1));
+    if (form_.sequential) {
+        LS_TRY(upload_norm(f, p + "norm1b", L.norm1b));
+        LS_TRY(upload_vector(f, p + "canon1", (int64_t)W * taps_, &L.canon1));
+    }
+    LS_TRY(upload_mixer(f, p, i, L));
     if (L.has_mlp) {
-        MoeFeedForward& M = L.mlp;
-        LS_TRY(upload_vector(f, p + "norm2", W, &L.norm2));
-        LS_TRY(upload_vector(f, p + "mlp.router", (int64_t)M.experts * W, &M.router));
-        std::vector<std::string> gu, dn;
-        for (int e = 0; e < M.experts; ++e) {
-            const std::string q = p + "mlp.e" + std::to_string(e) + ".";
-            gu.push_back(q + "gate"); gu.push_back(q + "up"); dn.push_back(q + "down");
+        LS_TRY(upload_norm(f, p + "norm2", L.norm2));
+        if (form_.sequential) {
+            LS_TRY(upload_norm(f, p + "norm2b", L.norm2b));
+            LS_TRY(upload_vector(f, p + "canon2", (int64_t)W * taps_, &L.canon2));
         }
-        LS_TRY(upload_matrix(f, gu, W, M.routed.gate_up, M.experts));
-        LS_TRY(upload_matrix(f, dn, M.routed.ff, M.routed.down, M.experts));
-        if (M.routed.gate_up.out_f != 2 * M.routed.ff || M.routed.down.out_f != W) return fail(NTK_E_SHAPE, "layer " + std::to_string(i) + ": expert matrices do not have the configured sizes");
-        if (M.has_shared) {
-            LS_TRY(upload_matrix(f, {p + "mlp.shared.gate", p + "mlp.shared.up"}, W, M.shared.gate_up));
-            LS_TRY(upload_matrix(f, {p + "mlp.shared.down"}, M.shared.ff, M.shared.down));
-            if (M.shared.gate_up.out_f != 2 * M.shared.ff || M.shared.down.out_f != W) return fail(NTK_E_SHAPE, "layer " + std::to_string(i) + ": shared expert matrices do not have the configured sizes");
-            LS_TRY(upload_vector(f, p + "mlp.shared.sg", W, &M.shared_gate));
-        }
+        LS_TRY(upload_mlp(f, p, i, L));
     }
     return NTK_OK;
 }
@@ -262,8 +446,8 @@ int LayerStackModel::load(const std::string& dir, const SeqLoadOptions& opt) {
     LS_TRY(upload_matrix(f, {"embed"}, W, embed_));
     LS_TRY(upload_matrix(f, {"head"}, W, head_));
     if (embed_.out_f != info_.vocab || head_.out_f != info_.vocab) return fail(NTK_E_SHAPE, "embed / head do not have 'vocab' rows");
-    LS_TRY(upload_vector(f, "final.norm", W, &final_norm_));
-    if (has_loop_) {
+    LS_TRY(upload_norm(f, "final.norm", final_norm_));
+    if (has_loop_ && form_.loop_projection) {
         LS_TRY(upload_matrix(f, {"loop.in"}, 2 * W, loop_in_));
         if (loop_in_.out_f != W) return fail(NTK_E_SHAPE, "tensor 'loop.in' is not [width, 2 width]");
     }
@@ -276,36 +460,51 @@ int LayerStackModel::load(const std::string& dir, const SeqLoadOptions& opt) {
 int LayerStackModel::alloc_buffers() {
     const int W = info_.width;
     chunk_ = std::min(opt_.max_context, 1024);
+    size_t sc = 0, wsc = 0;
     for (const auto& L : layers_) {
-        const LatentMixer& m = L.mix;
-        max_in_ = std::max<int>(max_in_, (int)m.in.out_f);
-        max_qrank_ = std::max(max_qrank_, m.q_rank);
-        max_hqd_ = std::max(max_hqd_, m.heads * m.qd());
-        max_hdv_ = std::max(max_hdv_, m.heads * m.vdim);
-        max_hdn_ = std::max(max_hdn_, m.heads * m.dim);
-        max_fold_ = std::max(max_fold_, m.heads * m.row());
-        max_hr_ = std::max(max_hr_, m.heads * m.kv_rank);
-        if (m.kv_rank > 512 || m.vdim > 512) return fail(NTK_E_SHAPE, "kv_rank and vdim up to 512 are supported");
-        if (L.has_mlp) {
+        if (L.mixer == kMixLatent) {
+            const LatentMixer& m = L.mix;
+            max_in_ = std::max<int>(max_in_, (int)m.in.out_f);
+            max_qrank_ = std::max(max_qrank_, m.q_rank);
+            max_hqd_ = std::max(max_hqd_, m.heads * m.qd());
+            max_hdv_ = std::max(max_hdv_, m.heads * m.vdim);
+            max_hdn_ = std::max(max_hdn_, m.heads * m.dim);
+            max_fold_ = std::max(max_fold_, m.heads * m.row());
+            max_hr_ = std::max(max_hr_, m.heads * m.kv_rank);
+            if (m.kv_rank > 512 || m.vdim > 512) return fail(NTK_E_SHAPE, "kv_rank and vdim up to 512 are supported");
+            sc = std::max(sc, ntk_latent_attention_scratch(kSharedRows, m.heads, m.kv_rank, opt_.max_context));
+        } else if (L.mixer == kMixWindow) {
+            const WindowMixer& m = L.att;
+            max_in_ = std::max<int>(max_in_, (int)m.in.out_f);
+            max_hdv_ = std::max(max_hdv_, m.heads * m.vdim);
+            if (m.vdim > 512) return fail(NTK_E_SHAPE, "vdim up to 512 is supported");
+            wsc = std::max(wsc, ntk_window_attention_scratch(chunk_, m.heads, m.maps, m.vdim, opt_.max_context));
+        } else {
+            const LightningMixer& m = L.lin;
+            max_in_ = std::max<int>(max_in_, (int)m.in.out_f);
+            max_hdv_ = std::max(max_hdv_, m.heads * m.vdim);
+        }
+        if (L.mlp_kind == kMlpMoe) {
             max_top_ = std::max(max_top_, L.mlp.top);
             max_e_ = std::max(max_e_, L.mlp.experts);
             max_ff2_ = std::max(max_ff2_, 2 * L.mlp.routed.ff);
             if (L.mlp.has_shared) max_sff2_ = std::max(max_sff2_, 2 * L.mlp.shared.ff);
+        } else if (L.mlp_kind == kMlpDense) {
+            max_ffn_ = std::max(max_ffn_, L.ffn.ff);
         }
     }
     const size_t C = (size_t)chunk_, ctx = (size_t)opt_.max_context;
-    auto fl = [&](float** p, size_t n) { *p = (float*)dev_alloc(n * sizeof(float)); return *p != nullptr; };
+    auto fl = [&](float** p, size_t n) { *p = (float*)dev_alloc(std::max<size_t>(n, 1) * sizeof(float)); return *p != nullptr; };
     auto in = [&](int** p, size_t n) { *p = (int*)dev_alloc(n * sizeof(int)); return *p != nullptr; };
-    bool ok = fl(&x_, C * W) && fl(&x0_, C * W) && fl(&cat_, C * 2 * W) && fl(&h1_, C * W) && fl(&h2_, C * W) && fl(&a_, C * max_in_) &&
-              fl(&cq_, C * std::max(max_qrank_, 1)) && fl(&q_, C * max_hqd_) && fl(&qf_, (size_t)kSharedRows * max_fold_) && fl(&lat_, (size_t)kSharedRows * max_hr_) &&
-              fl(&att_, C * max_hdv_) && fl(&kx_, ctx * max_hdn_) && fl(&vx_, ctx * max_hdv_) && fl(&mix_, C * W) && fl(&xw_, C * W) && fl(&hn_, C * W) &&
-              in(&tokens_dev_, 2 * C);
+    bool ok = fl(&x_, C * W) && fl(&x0_, C * W) && fl(&h1_, C * W) && fl(&h2_, C * W) && fl(&a_, C * max_in_) && fl(&att_, C * max_hdv_) && fl(&mix_, C * W) &&
+              fl(&xw_, C * W) && fl(&hn_, C * W) && in(&tokens_dev_, 2 * C);
+    if (max_hqd_ > 0)      // latent mixers: query latents, folded queries, the up-projected keys and values of the visible range
+        ok = ok && fl(&cat_, C * 2 * W) && fl(&cq_, C * std::max(max_qrank_, 1)) && fl(&q_, C * max_hqd_) && fl(&qf_, (size_t)kSharedRows * max_fold_) &&
+             fl(&lat_, (size_t)kSharedRows * max_hr_) && fl(&kx_, ctx * max_hdn_) && fl(&vx_, ctx * max_hdv_) && fl(&scratch_, sc);
+    if (form_.sequential) ok = ok && fl(&hist_, (C + (size_t)taps_ - 1) * W) && fl(&ff_, C * W) && fl(&zf_, C * max_ffn_) && fl(&wscratch_, wsc);
     want_dev_ = tokens_dev_ ? tokens_dev_ + C : nullptr;   // one staging area: [tokens of a pass | wanted places], filled by ONE stream-ordered copy from pinned memory
     h_stage_ = (int*)nt_hip_malloc_host(2 * C * sizeof(int));
     ok = ok && h_stage_ != nullptr;
-    size_t sc = 0;
-    for (const auto& L : layers_) sc = std::max(sc, ntk_latent_attention_scratch(kSharedRows, L.mix.heads, L.mix.kv_rank, opt_.max_context));
-    ok = ok && fl(&scratch_, sc);
     if (max_top_ > 0) {
         const size_t P = C * max_top_;
         ok = ok && in(&ids_, P) && fl(&wts_, P) && fl(&sg_, C) && in(&offsets_, (size_t)max_e_ + 1) && in(&order_, P) && in(&where_, P) && fl(&gu_, P * max_ff2_) &&
@@ -313,10 +512,22 @@ int LayerStackModel::alloc_buffers() {
         if (max_sff2_ > 0) ok = ok && fl(&sgu_, C * max_sff2_) && fl(&sact_, C * (max_sff2_ / 2)) && fl(&sdn_, C * W);
     }
     if (!ok) return fail(NTK_E_NOMEM, "out of device memory (activation buffers)");
+    // what every slot holds per layer run: cache rows per position, the recurrent state, the convolutions' last inputs (mixer's, then feed-forward's)
     for (auto& r : runs_) {
-        const size_t row = (size_t)layers_[(size_t)r.layer].mix.row();
-        r.cache = (float*)dev_alloc((size_t)opt_.slots * ctx * row * sizeof(float));
-        if (!r.cache) return fail(NTK_E_NOMEM, "out of device memory (cache)");
+        const StackLayer& L = layers_[(size_t)r.layer];
+        const size_t row = (size_t)L.cache_row();
+        if (row) {
+            r.cache = (float*)dev_alloc((size_t)opt_.slots * ctx * row * sizeof(float));
+            if (!r.cache) return fail(NTK_E_NOMEM, "out of device memory (cache)");
+        }
+        if (L.mixer == kMixLightning) {
+            r.state = (float*)dev_alloc((size_t)opt_.slots * L.lin.state_floats() * sizeof(float));
+            if (!r.state) return fail(NTK_E_NOMEM, "out of device memory (state)");
+        }
+        if (form_.sequential && taps_ > 1) {
+            r.conv = (float*)dev_alloc((size_t)opt_.slots * 2 * (taps_ - 1) * W * sizeof(float));
+            if (!r.conv) return fail(NTK_E_NOMEM, "out of device memory (state)");
+        }
     }
     return NTK_OK;
 }
@@ -326,6 +537,8 @@ int LayerStackModel::acquire_slot() { const int s = slots_.acquire(); return s <
 int LayerStackModel::release_slot(int slot) { return slots_.release(slot) ? NTK_OK : NTK_E_SHAPE; }
 int LayerStackModel::truncate_slot(int slot, int length) {
     if (!slots_.live(slot) || length < 0 || length > slots_.length(slot)) return NTK_E_SHAPE;
+    // a recurrent state or a convolution's last inputs cannot be rolled back: such a sequence restarts (position 0 reads no state) or stays
+    if (has_state_ && length != 0 && length != slots_.length(slot)) return fail(NTK_E_SHAPE, "truncate: a model with recurrent state can only be cut back to its start");
     slots_.set_length(slot, length);
     return NTK_OK;
 }
@@ -338,7 +551,7 @@ int LayerStackModel::run_mixer(const StackLayer& L, float* cache, int T, int pos
     const bool few = T <= ntk_dense_few_rows();
     ntk_dense_desc d{};
     d.Y = a_; d.ldy = na; d.X = few ? x_ : h1_; d.ldx = W; d.W = m.in.ptr; d.wdtype = m.in.dtype; d.G = 1; d.row_div = 1; d.T = T; d.N = na; d.K = W;
-    if (few) { d.norm_w = L.norm1; d.norm_eps = eps_; d.norm_offset = 1.0f; }
+    if (few) { d.norm_w = L.norm1.w; d.norm_eps = eps_; d.norm_offset = 1.0f; }
     LS_TRY(ntk_dense(&d, stream_));
     float* q = a_;
     int ldq = na;
@@ -369,38 +582,110 @@ int LayerStackModel::run_mixer(const StackLayer& L, float* cache, int T, int pos
     return ntk_dense_linear(mix_, W, att_, hv, m.o.ptr, m.o.dtype, T, W, hv, 0, stream_);
 }
 
-int LayerStackModel::run_experts(const ClippedExperts& ex, const float* h, float* gu, float* act, float* out, int rows, const int* offsets, const int* order, int top) {
+// the window mixer: one product for [q | k | v], rotation and cache rows, attention over the window, output projection -> mix_
+int LayerStackModel::run_window(const StackLayer& L, float* cache, int T, int pos0) {
+    const WindowMixer& m = L.att;
+    const int W = info_.width, na = (int)m.in.out_f, hv = m.heads * m.vdim;
+    LS_TRY(ntk_dense_linear(a_, na, h1_, W, m.in.ptr, m.in.dtype, T, na, W, 0, stream_));
+    ntk_rotary rot{m.rot_freq, 1.0f, m.rot_dims};
+    LS_TRY(ntk_window_prepare(cache, m.row(), a_, na, a_ + m.k_off, na, a_ + m.v_off, na, m.heads, m.kv_heads, m.maps, m.dim, m.vdim, &rot, pos0, T, stream_));
+    ntk_window_attention_desc d{};
+    d.out = att_; d.ldo = hv; d.q = a_; d.ldq = na; d.cache = cache; d.row = m.row(); d.H = m.heads; d.G = m.kv_heads; d.maps = m.maps; d.dn = m.dim; d.dv = m.vdim;
+    d.pos0 = pos0; d.T = T; d.window = m.window; d.scale = m.scale; d.lambda = m.lambda;
+    d.sub_norm = m.maps == 2 ? 1 : 0; d.eps = eps_; d.out_scale = m.maps == 2 ? 1.0f - m.diff : 1.0f;
+    d.scratch = wscratch_;
+    LS_TRY(ntk_window_attention(&d, stream_));
+    return ntk_dense_linear(mix_, W, att_, hv, m.o.ptr, m.o.dtype, T, W, hv, 0, stream_);
+}
+
+// the lightning mixer: one product for [q | k | v | gate], the recurrence (silu on the way in), gated RMS norm over the joined heads, output projection -> mix_
+int LayerStackModel::run_lightning(const StackLayer& L, float* state, int T, int pos0) {
+    const LightningMixer& m = L.lin;
+    const int W = info_.width, na = (int)m.in.out_f, hv = m.heads * m.vdim;
+    LS_TRY(ntk_dense_linear(a_, na, h1_, W, m.in.ptr, m.in.dtype, T, na, W, 0, stream_));
+    LS_TRY(ntk_lightning_attention(att_, hv, a_, na, a_ + m.k_off, na, a_ + m.v_off, na, m.log_decay, state, m.heads, m.dim, m.vdim, 1, pos0, T, stream_));
+    LS_TRY(ntk_gated_rmsnorm(att_, hv, att_, hv, m.norm, a_ + m.g_off, na, T, hv, eps_, stream_));
+    return ntk_dense_linear(mix_, W, att_, hv, m.o.ptr, m.o.dtype, T, W, hv, 0, stream_);
+}
+
+int LayerStackModel::run_experts(const MoeFeedForward& M, const GatedExperts& ex, const float* h, float* gu, float* act, float* out, int rows, const int* offsets, const int* order, int top) {
     const int W = info_.width;
     ntk_dense_desc d{};
     d.Y = gu; d.ldy = 2 * ex.ff; d.X = h; d.ldx = W; d.W = ex.gate_up.ptr; d.wstride = ex.gate_up.stride(); d.wdtype = ex.gate_up.dtype;
     d.offsets = offsets; d.G = ex.gate_up.count; d.rows = order; d.row_div = top; d.T = rows; d.N = 2 * ex.ff; d.K = W; d.accumulate = 0;
     if (rows <= ntk_dense_few_rows()) {   // decoding: the activation inside the product's launch
-        d.Y = act; d.ldy = ex.ff; d.glu_ff = ex.ff; d.glu_limit = ex.limit; d.glu_alpha = kGluAlpha;
+        d.Y = act; d.ldy = ex.ff; d.glu_ff = ex.ff; d.glu_limit = ex.limit; d.glu_alpha = M.glu_alpha; d.glu_up_offset = M.glu_up_offset;
         LS_TRY(ntk_dense(&d, stream_));
         d.glu_ff = 0;
     } else {
         LS_TRY(ntk_dense(&d, stream_));
-        LS_TRY(ntk_clipped_glu(act, gu, rows, ex.ff, ex.limit, kGluAlpha, stream_));
+        LS_TRY(ntk_glu(act, gu, rows, ex.ff, ex.limit, M.glu_alpha, M.glu_up_offset, stream_));
     }
     d.Y = out; d.ldy = W; d.X = act; d.ldx = ex.ff; d.W = ex.down.ptr; d.wstride = ex.down.stride(); d.wdtype = ex.down.dtype;
     d.rows = nullptr; d.row_div = 1; d.N = W; d.K = ex.ff;
     return ntk_dense(&d, stream_);
 }
 
-int LayerStackModel::run_moe(const StackLayer& L, int T) {
+// router, grouping, the experts' products; then either straight into the stream together with the mixer's output (parallel form) or as a sum of its own
+// in ff_ (sequential form: it is normed before it joins the stream)
+int LayerStackModel::run_moe(const StackLayer& L, int T, bool into_stream) {
     const MoeFeedForward& M = L.mlp;
     const int W = info_.width;
-    LS_TRY(ntk_moe_route(ids_, wts_, M.has_shared ? sg_ : nullptr, h2_, W, M.router, M.has_shared ? M.shared_gate : nullptr, T, W, M.experts, M.top, stream_));
+    float* sgate = M.has_shared && M.shared_gate ? sg_ : nullptr;
+    LS_TRY(ntk_moe_route_ex(ids_, wts_, sgate, h2_, W, M.router, sgate ? M.shared_gate : nullptr, T, W, M.experts, M.top, &M.route, stream_));
     LS_TRY(ntk_moe_group(offsets_, order_, where_, ids_, T, M.top, M.experts, stream_));
-    LS_TRY(run_experts(M.routed, h2_, gu_, act_, dn_, T * M.top, offsets_, order_, M.top));
-    if (M.has_shared) LS_TRY(run_experts(M.shared, h2_, sgu_, sact_, sdn_, T, nullptr, nullptr, 1));
-    // stream += mixer + sum of the chosen experts + gated shared expert
-    return ntk_moe_combine(x_, mix_, dn_, where_, wts_, M.has_shared ? sdn_ : nullptr, M.has_shared ? sg_ : nullptr, T, M.top, W, stream_);
+    LS_TRY(run_experts(M, M.routed, h2_, gu_, act_, dn_, T * M.top, offsets_, order_, M.top));
+    if (M.has_shared) LS_TRY(run_experts(M, M.shared, h2_, sgu_, sact_, sdn_, T, nullptr, nullptr, 1));
+    if (into_stream) return ntk_moe_combine(x_, mix_, dn_, where_, wts_, M.has_shared ? sdn_ : nullptr, sgate, T, M.top, W, stream_);
+    return ntk_moe_sum(ff_, dn_, where_, wts_, M.has_shared ? sdn_ : nullptr, sgate, T, M.top, W, stream_);
+}
+
+// up, the polynomial activation over every token's row of ff values, down -> ff_ (the activation runs in place in the up product's buffer)
+int LayerStackModel::run_dense_ff(const StackLayer& L, int T) {
+    const DenseFeedForward& D = L.ffn;
+    const int W = info_.width;
+    LS_TRY(ntk_dense_linear(zf_, D.ff, h2_, W, D.up.ptr, D.up.dtype, T, D.ff, W, 0, stream_));
+    LS_TRY(ntk_polynorm(zf_, D.ff, zf_, D.ff, D.act, T, D.ff, eps_, stream_));
+    return ntk_dense_linear(ff_, W, zf_, D.ff, D.down.ptr, D.down.dtype, T, W, D.ff, 0, stream_);
+}
+
+// out = h + conv(h), h = layer norm of the stream: the carried inputs in front of the portion's, the convolution, and the portion's last inputs carried on
+int LayerStackModel::norm_conv(const NormW& nw, const float* canon, float* conv_state, float* out, int T, int pos0) {
+    const int W = info_.width;
+    LS_TRY(ntk_layernorm_history(hist_, x_, W, nw.w, nw.b, conv_state, taps_, pos0, T, W, eps_, stream_));
+    return ntk_causal_conv_mix(out, W, hist_, canon, conv_state, taps_, T, W, stream_);
+}
+
+int LayerStackModel::sequential_layer(const Run& run, const StackLayer& L, int slot, int T, int pos0) {
+    const int W = info_.width;
+    float* conv = run.conv ? run.conv + (size_t)slot * 2 * (taps_ - 1) * W : nullptr;
+    LS_TRY(norm_conv(L.norm1, L.canon1, conv, h1_, T, pos0));
+    if (L.mixer == kMixWindow) LS_TRY(run_window(L, run.cache + (size_t)slot * opt_.max_context * L.att.row(), T, pos0));
+    else LS_TRY(run_lightning(L, run.state + (size_t)slot * L.lin.state_floats(), T, pos0));
+    LS_TRY(ntk_layernorm(x_, W, mix_, W, L.norm1b.w, L.norm1b.b, T, W, eps_, 1, stream_));
+    if (!L.has_mlp) return NTK_OK;
+    LS_TRY(norm_conv(L.norm2, L.canon2, conv ? conv + (size_t)(taps_ - 1) * W : nullptr, h2_, T, pos0));
+    if (L.mlp_kind == kMlpMoe) LS_TRY(run_moe(L, T, false));
+    else LS_TRY(run_dense_ff(L, T));
+    return ntk_layernorm(x_, W, ff_, W, L.norm2b.w, L.norm2b.b, T, W, eps_, 1, stream_);
+}
+
+int LayerStackModel::parallel_layer(const Run& run, const StackLayer& L, int slot, int T, int pos0) {
+    const int W = info_.width;
+    if (T > ntk_dense_few_rows()) {
+        LS_TRY(ntk_rmsnorm_offset(h1_, L.norm1.w, L.has_mlp ? h2_ : nullptr, L.has_mlp ? L.norm2.w : nullptr, W, x_, W, T, W, eps_, 1.0f, stream_));
+    } else if (L.has_mlp) {   // decoding: the mixer's norm runs inside its first product (run_mixer); the feed-forward's input has three readers
+        LS_TRY(ntk_rmsnorm_offset(h2_, L.norm2.w, nullptr, nullptr, W, x_, W, T, W, eps_, 1.0f, stream_));
+    }
+    float* cache = run.cache + (size_t)slot * opt_.max_context * L.mix.row();
+    LS_TRY(run_mixer(L, cache, T, pos0));
+    if (L.has_mlp) return run_moe(L, T, true);
+    return ntk_residual_add(x_, mix_, nullptr, T * W, stream_);
 }
 
 int LayerStackModel::portion(int slot, const int* tokens_dev, int T, int pos0, const int* want_dev, int n_want, float* logits_out) {
     const int W = info_.width;
-    LS_TRY(ntk_embed_dense(x0_, embed_.ptr, embed_.dtype, tokens_dev, T, info_.vocab, W, stream_));
+    LS_TRY(ntk_embed_dense_scaled(x0_, embed_.ptr, embed_.dtype, tokens_dev, T, info_.vocab, W, embed_scale_, stream_));
     bool x_is_x0 = true;   // until the first layer run writes x_
     for (size_t r = 0; r < runs_.size(); ++r) {
         const Run& run = runs_[r];
@@ -411,15 +696,8 @@ int LayerStackModel::portion(int slot, const int* tokens_dev, int T, int pos0, c
             LS_TRY(ntk_dense_linear(x_, W, cat_, 2 * W, loop_in_.ptr, loop_in_.dtype, T, W, 2 * W, 0, stream_));
             x_is_x0 = false;
         }
-        if (T > ntk_dense_few_rows()) {
-            LS_TRY(ntk_rmsnorm_offset(h1_, L.norm1, L.has_mlp ? h2_ : nullptr, L.has_mlp ? L.norm2 : nullptr, W, x_, W, T, W, eps_, 1.0f, stream_));
-        } else if (L.has_mlp) {   // decoding: the mixer's norm runs inside its first product (run_mixer); the feed-forward's input has three readers
-            LS_TRY(ntk_rmsnorm_offset(h2_, L.norm2, nullptr, nullptr, W, x_, W, T, W, eps_, 1.0f, stream_));
-        }
-        float* cache = run.cache + (size_t)slot * opt_.max_context * L.mix.row();
-        LS_TRY(run_mixer(L, cache, T, pos0));
-        if (L.has_mlp) LS_TRY(run_moe(L, T));
-        else LS_TRY(ntk_residual_add(x_, mix_, nullptr, T * W, stream_));
+        if (form_.sequential) LS_TRY(sequential_layer(run, L, slot, T, pos0));
+        else LS_TRY(parallel_layer(run, L, slot, T, pos0));
         if (capture_ && capture_buf_) LS_TRY(ntk_rows_copy(capture_buf_ + r * (size_t)T * W, x_, (long long)T * W, stream_));
     }
     if (n_want > 0) {
@@ -430,9 +708,11 @@ int LayerStackModel::portion(int slot, const int* tokens_dev, int T, int pos0, c
         ntk_dense_desc d{};
         d.Y = logits_out; d.ldy = info_.vocab; d.X = rows; d.ldx = W; d.W = head_.ptr; d.wdtype = head_.dtype; d.G = 1; d.row_div = 1; d.T = n_want;
         d.N = info_.vocab; d.K = W;
-        if (n_want <= ntk_dense_few_rows()) { d.norm_w = final_norm_; d.norm_eps = eps_; d.norm_offset = 1.0f; }   // the output norm inside the head's launch
-        else { LS_TRY(ntk_rmsnorm_offset(hn_, final_norm_, nullptr, nullptr, W, rows, W, n_want, W, eps_, 1.0f, stream_)); d.X = hn_; }
+        if (final_norm_.b) { LS_TRY(ntk_layernorm(hn_, W, rows, W, final_norm_.w, final_norm_.b, n_want, W, eps_, 0, stream_)); d.X = hn_; }
+        else if (n_want <= ntk_dense_few_rows()) { d.norm_w = final_norm_.w; d.norm_eps = eps_; d.norm_offset = 1.0f; }   // the output norm inside the head's launch
+        else { LS_TRY(ntk_rmsnorm_offset(hn_, final_norm_.w, nullptr, nullptr, W, rows, W, n_want, W, eps_, 1.0f, stream_)); d.X = hn_; }
         LS_TRY(ntk_dense(&d, stream_));
+        if (logit_scale_ != 1.0f) LS_TRY(ntk_scale(logits_out, (long long)n_want * info_.vocab, logit_scale_, stream_));
     }
     return NTK_OK;
 }

@@ -1,13 +1,21 @@
 // engine/layer_stack.h -- model families described by a LIST of layers in config.json (type of mixer, its sizes, its feed-forward), with dense
-// bfloat16 weights in a safetensors file: a residual stream in F32, parallel layers (mixer and feed-forward read two norms of the same input), an
-// optional repeated span of layers (each pass with its own cache, entered through a projection of [stream ; embedding]), and an output norm + head.
+// bfloat16 weights in a safetensors file: a residual stream in F32, an optional repeated span of layers (each pass with its own cache and state), and an
+// output norm + head.  A family fixes the FORM of a layer (StackForm):
+//   parallel     x += mixer(norm1 x) + ff(norm2 x), RMS norms whose weight is stored around zero; the repeated span is entered through a projection
+//                of [stream ; embedding]                                                                                   -- "Fabolorn"
+//   sequential   x += norm1b(mixer(conv(norm1 x))), then x += norm2b(ff(conv(norm2 x))): layer norms with weight and bias before and after every
+//                sublayer, a short causal convolution added to every sublayer's input (its last inputs are part of a sequence's state), scaled
+//                embedding and logits                                                                                       -- "Nizorax"
 //
 // Mechanisms are parsed into parameter structs and run by the operators of include/ntk_layers.h, so another family can list them in another order
 // or with other constants:
 //   mixers        "latent_attention" (query through a normed latent, causal, optional frequency-scaled rotation) and "latent_attention_2" (query from
 //                 one matrix, sliding window): one LatentMixer each -- which of the options a layer has is read from its config keys;
-//   feed-forward  kind "moe": routed clipped-GLU experts + an optional gated shared expert.
-// Registered for the architecture "Fabolorn".
+//                 "attention": grouped-query attention over rotated keys with a sliding window, as a differential pair of score maps when the
+//                 config gives 'diff' (WindowMixer); "lightning": linear attention with a per-head decay and a recurrent state (LightningMixer);
+//   feed-forward  kind "moe": routed gated experts + an optional shared expert (MoeFeedForward: softmax or sigmoid scores, optional expert groups,
+//                 clipped or plain gated units); kind "dense": up, polynomial activation with unit-norm terms, down (DenseFeedForward).
+// What a sequence holds per layer run: cache rows per position (attention kinds), a recurrent state (lightning), the convolutions' last inputs.
 #pragma once
 #include <string>
 #include <vector>
@@ -41,33 +49,87 @@ struct LatentMixer {
     int row() const { return kv_rank + rot_dim; }
 };
 
-struct ClippedExperts {               // `count` experts of the same shape, stacked: gate rows then up rows, and the down matrices
+struct WindowMixer {                  // grouped-query attention, sliding window, one score map per head or a differential pair
+    int heads = 0, kv_heads = 0, dim = 0, vdim = 0, maps = 1;
+    int window = 0;                   // 0: causal over everything
+    float scale = 1.0f;
+    float diff = 0.0f, lambda = 0.0f; // maps == 2: out = (a_0 - lambda a_1) / rms * (1 - diff)
+    int rot_dims = 0;
+    double* rot_freq = nullptr;       // device [rot_dims / 2]
+    DenseW in;                        // rows [q | k | v] of one product over the mixer's input
+    int k_off = 0, v_off = 0;
+    DenseW o;
+    int row() const { return kv_heads * (maps * dim + vdim); }
+};
+
+struct LightningMixer {               // linear attention with a per-head decay; q, k, v through silu, gated RMS norm over the joined heads
+    int heads = 0, dim = 0, vdim = 0;
+    float* log_decay = nullptr;       // device F32 [heads]
+    DenseW in;                        // rows [q | k | v | gate]
+    int k_off = 0, v_off = 0, g_off = 0;
+    float* norm = nullptr;            // F32 [heads * vdim]
+    DenseW o;
+    size_t state_floats() const { return (size_t)heads * dim * vdim; }
+};
+
+struct GatedExperts {                 // `count` experts of the same shape, stacked: gate rows then up rows, and the down matrices
     int ff = 0;
-    float limit = 0.0f;
+    float limit = 0.0f;               // clamp of the gate (from above) and the up value (both sides); INFINITY: none
     DenseW gate_up, down;
 };
 
 struct MoeFeedForward {
     int experts = 0, top = 0;
+    ntk_route_desc route{};           // score function, expert groups, renormalisation, scale of the weights
+    float glu_alpha = 1.0f, glu_up_offset = 0.0f;   // act(g) = g * sigmoid(alpha g), multiplied by (up + offset)
     float* router = nullptr;          // F32 [experts][width]
-    ClippedExperts routed;
+    GatedExperts routed;
     bool has_shared = false;
-    ClippedExperts shared;
-    float* shared_gate = nullptr;     // F32 [width]
+    GatedExperts shared;
+    float* shared_gate = nullptr;     // F32 [width]; none: the shared expert is added as it is
 };
+
+struct DenseFeedForward {             // down(act(up h)), act = a N(z) + b N(z^2) + c N(z^3) + e
+    int ff = 0;
+    DenseW up, down;
+    float* act = nullptr;             // F32 [4]
+};
+
+struct NormW { float* w = nullptr; float* b = nullptr; };   // b: layer norm with bias (sequential form); none: RMS norm, weight around zero
+
+enum MixerKind { kMixLatent = 0, kMixWindow = 1, kMixLightning = 2 };
+enum MlpKind { kMlpNone = 0, kMlpMoe = 1, kMlpDense = 2 };
 
 struct StackLayer {
     std::string type;
-    float* norm1 = nullptr;
-    float* norm2 = nullptr;
+    int mixer = kMixLatent;
+    NormW norm1, norm2, norm1b, norm2b;     // (1b, 2b: the norms after a sublayer, sequential form)
+    float* canon1 = nullptr;                // F32 [width][taps]: the convolution on the mixer's input
+    float* canon2 = nullptr;                // ... on the feed-forward's input
     LatentMixer mix;
+    WindowMixer att;
+    LightningMixer lin;
+    int mlp_kind = kMlpNone;
     bool has_mlp = false;
     MoeFeedForward mlp;
+    DenseFeedForward ffn;
+    int cache_row() const { return mixer == kMixLatent ? mix.row() : mixer == kMixWindow ? att.row() : 0; }
+};
+
+// what a family fixes about its layers (everything else is read from config.json)
+struct StackForm {
+    bool sequential = false;          // see the head of this file
+    bool loop_projection = true;      // the repeated span is entered through 'loop.in' over [stream ; embedding]
+    int router_score = 0;             // 0 softmax, 1 sigmoid
+    bool router_renorm = true;
+    bool clipped_glu = true;          // experts: clipped gated unit with slope kGluAlpha and up + 1; else silu(gate) * up
+    bool shared_gate = true;          // the shared expert sits behind a per-token sigmoid gate
+    int group_top = 2;                // a group's score: the sum of this many of its largest scores
 };
 
 class LayerStackModel : public SequenceModel {
 public:
-    LayerStackModel() = default;
+    explicit LayerStackModel(const StackForm& form) : form_(form) {}
     ~LayerStackModel() override;
     int load(const std::string& dir, const SeqLoadOptions& opt) override;
     const SeqModelInfo& info() const override { return info_; }
@@ -86,10 +148,16 @@ public:
     static constexpr int kSharedRows = 8;     // up to this many tokens per portion take the decode form of the mixer (and the GEMV form of the products)
 
 private:
-    struct Run { int layer; bool enters; float* cache; };
+    struct Run { int layer; bool enters; float* cache; float* state; float* conv; };   // per slot: cache rows, recurrent state, [2][taps - 1][width] last inputs
     int fail(int st, const std::string& why) { err_ = why; return st; }
     int parse(const ModelFolder& f);
     int parse_mixer(const Json& L, const std::string& type, LatentMixer& m);
+    int parse_window(const Json& L, WindowMixer& m);
+    int parse_lightning(const Json& L, LightningMixer& m);
+    int parse_mlp(const Json& ml, const std::string& where, StackLayer& S);
+    int upload_norm(const ModelFolder& f, const std::string& name, NormW& out);
+    int upload_mixer(const ModelFolder& f, const std::string& p, int i, StackLayer& L);
+    int upload_mlp(const ModelFolder& f, const std::string& p, int i, StackLayer& L);
     int upload_layer(const ModelFolder& f, int i, StackLayer& L);
     int upload_vector(const ModelFolder& f, const std::string& name, int64_t n, float** out);
     int upload_matrix(const ModelFolder& f, const std::vector<std::string>& names, int64_t in_f, DenseW& out, int count = 1);
@@ -97,30 +165,40 @@ private:
     void* dev_alloc(size_t bytes);
     int portion(int slot, const int* tokens_dev, int T, int pos0, const int* want_dev, int n_want, float* logits_out);
     int run_mixer(const StackLayer& L, float* cache, int T, int pos0);
-    int run_moe(const StackLayer& L, int T);
-    int run_experts(const ClippedExperts& ex, const float* h, float* gu, float* act, float* out, int rows, const int* offsets, const int* order, int top);
+    int run_window(const StackLayer& L, float* cache, int T, int pos0);
+    int run_lightning(const StackLayer& L, float* state, int T, int pos0);
+    int run_moe(const StackLayer& L, int T, bool into_stream);
+    int run_dense_ff(const StackLayer& L, int T);
+    int run_experts(const MoeFeedForward& M, const GatedExperts& ex, const float* h, float* gu, float* act, float* out, int rows, const int* offsets, const int* order, int top);
+    int norm_conv(const NormW& nw, const float* canon, float* conv_state, float* out, int T, int pos0);
+    int sequential_layer(const Run& run, const StackLayer& L, int slot, int T, int pos0);
+    int parallel_layer(const Run& run, const StackLayer& L, int slot, int T, int pos0);
 
+    StackForm form_;
     SeqModelInfo info_;
     std::string err_;
     SeqLoadOptions opt_;
     int wdtype_ = NTK_DT_BF16;
     float eps_ = 1e-6f;
+    int taps_ = 1;                    // the input convolutions' taps (sequential form)
+    float embed_scale_ = 1.0f, logit_scale_ = 1.0f;
+    bool has_state_ = false;          // some layer carries a recurrent state or convolution inputs: a slot can only be cut back to its start
     std::vector<StackLayer> layers_;
     std::vector<Run> runs_;
     bool has_loop_ = false;
     DenseW embed_, head_, loop_in_;
-    float* final_norm_ = nullptr;
+    NormW final_norm_;
     uint64_t weight_bytes_ = 0;
     std::vector<void*> allocs_;
     SlotTable slots_;
     void* stream_ = nullptr;
     int chunk_ = 0;                   // tokens per internal portion
     // maxima over the layers (buffer sizes)
-    int max_in_ = 0, max_qrank_ = 0, max_hqd_ = 0, max_hdv_ = 0, max_hdn_ = 0, max_fold_ = 0, max_hr_ = 0, max_top_ = 0, max_e_ = 0, max_ff2_ = 0, max_sff2_ = 0;
+    int max_ffn_ = 0, max_in_ = 0, max_qrank_ = 0, max_hqd_ = 0, max_hdv_ = 0, max_hdn_ = 0, max_fold_ = 0, max_hr_ = 0, max_top_ = 0, max_e_ = 0, max_ff2_ = 0, max_sff2_ = 0;
     // activations
     float *x_ = nullptr, *x0_ = nullptr, *cat_ = nullptr, *h1_ = nullptr, *h2_ = nullptr, *a_ = nullptr, *cq_ = nullptr, *q_ = nullptr, *qf_ = nullptr, *lat_ = nullptr,
           *att_ = nullptr, *kx_ = nullptr, *vx_ = nullptr, *mix_ = nullptr, *wts_ = nullptr, *sg_ = nullptr, *gu_ = nullptr, *act_ = nullptr, *dn_ = nullptr,
-          *sgu_ = nullptr, *sact_ = nullptr, *sdn_ = nullptr, *scratch_ = nullptr, *xw_ = nullptr, *hn_ = nullptr;
+          *sgu_ = nullptr, *sact_ = nullptr, *sdn_ = nullptr, *scratch_ = nullptr, *xw_ = nullptr, *hn_ = nullptr, *hist_ = nullptr, *ff_ = nullptr, *zf_ = nullptr, *wscratch_ = nullptr;
     int *ids_ = nullptr, *offsets_ = nullptr, *order_ = nullptr, *where_ = nullptr, *tokens_dev_ = nullptr, *want_dev_ = nullptr;
     int* h_stage_ = nullptr;          // pinned: tokens and wanted places of the pass being launched
     float* logits_ = nullptr;

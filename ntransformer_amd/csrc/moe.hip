@@ -14,8 +14,25 @@ constexpr int kMaxExperts = 256;
 // one workgroup per token: its 16 waves share the experts (wave w: experts w, w + 16, ...), a lane requests its whole part of the router row before
 // it uses any of it; thread 0 then does the softmax and the `top` picks over the scores in LDS
 constexpr int kRouteThreads = 1024;
+struct RouteForm { int score, groups, keep, group_top, renorm; float scale; };
+
+// the largest of a wave's 4 x 64 values (lane l holds entries l, l + 64, l + 128, l + 192); equal values: the lower index
+__device__ __forceinline__ void wave_argmax4(const float (&v)[4], int lane, float& bv, int& bi) {
+    bv = v[0];
+    bi = lane;
+#pragma unroll
+    for (int c = 1; c < 4; ++c)
+        if (v[c] > bv) { bv = v[c]; bi = lane + 64 * c; }      // (equal values: the lower index stays)
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, 64);
+        const int oi = __shfl_xor(bi, o, 64);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+}
+
 __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(int* ids, float* wts, float* sgate, const float* h, int ldh, const float* wr, const float* wsg,
-                                                                 int n, int E, int top) {
+                                                                 int n, int E, int top, const RouteForm f) {
     __shared__ float z[kMaxExperts];
     extern __shared__ __attribute__((aligned(16))) float xs[];   // the token's row
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = kRouteThreads / 64;
@@ -44,38 +61,82 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(int* ids, floa
     }
     __syncthreads();
     if (wave != 0) return;
-    // softmax and the picks by one wave: lane l holds experts l, l + 64, l + 128, l + 192
+    // scores and the picks by one wave: lane l holds experts l, l + 64, l + 128, l + 192
     float v[4];
-    float m = -INFINITY;
+    float den = 1.0f;
+    if (f.score == 0) {
+        float m = -INFINITY;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) { v[c] = lane + 64 * c < E ? z[lane + 64 * c] : -INFINITY; m = fmaxf(m, v[c]); }
-    m = wave_max(m);
-    float den = 0.0f;
+        for (int c = 0; c < 4; ++c) { v[c] = lane + 64 * c < E ? z[lane + 64 * c] : -INFINITY; m = fmaxf(m, v[c]); }
+        m = wave_max(m);
+        den = 0.0f;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) { v[c] = lane + 64 * c < E ? expf(v[c] - m) : -1.0f; den += fmaxf(v[c], 0.0f); }
-    den = wave_sum(den);
+        for (int c = 0; c < 4; ++c) { v[c] = lane + 64 * c < E ? expf(v[c] - m) : -1.0f; den += fmaxf(v[c], 0.0f); }
+        den = wave_sum(den);
+    } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[c] = lane + 64 * c < E ? 1.0f / (1.0f + expf(-z[lane + 64 * c])) : -1.0f;
+    }
     __shared__ int pick_id[kMaxExperts];
     __shared__ float pick_sc[kMaxExperts];
+    if (f.groups > 1) {
+        // group scores: lane l owns groups l, l + 64, ...: the sum of the group's `group_top` largest scores (scores are >= 0; taken ones are marked -1)
+        __shared__ float sc[kMaxExperts];
+        __shared__ unsigned char open_group[kMaxExperts];
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            if (lane + 64 * c < E) sc[lane + 64 * c] = v[c];
+        __builtin_amdgcn_wave_barrier();
+        const int per = E / f.groups;
+        float gs[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int g = lane + 64 * c;
+            gs[c] = -1.0f;
+            if (g < f.groups) {
+                float sum = 0.0f;
+                int taken[8];
+                const int nt = min(min(f.group_top, per), 8);
+                for (int k = 0; k < nt; ++k) {
+                    float best = -1.0f;
+                    int bi = -1;
+                    for (int e = g * per; e < (g + 1) * per; ++e) {
+                        bool used = false;
+                        for (int u = 0; u < k; ++u) used = used || taken[u] == e;
+                        if (!used && sc[e] > best) { best = sc[e]; bi = e; }
+                    }
+                    taken[k] = bi;
+                    sum += best;
+                }
+                gs[c] = sum;
+            }
+            if (g < kMaxExperts) open_group[g] = 0;
+        }
+        __builtin_amdgcn_wave_barrier();
+        for (int k = 0; k < f.keep; ++k) {
+            float bv;
+            int bi;
+            wave_argmax4(gs, lane, bv, bi);
+            if (lane == 0) open_group[bi] = 1;
+            if ((bi & 63) == lane) gs[bi >> 6] = -2.0f;
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            if (lane + 64 * c < E && !open_group[(lane + 64 * c) / per]) v[c] = -1.0f;
+    }
     float chosen = 0.0f;
     for (int s = 0; s < top; ++s) {
-        float bv = v[0];
-        int bi = lane;
-#pragma unroll
-        for (int c = 1; c < 4; ++c)
-            if (v[c] > bv) { bv = v[c]; bi = lane + 64 * c; }      // (equal values: the lower index stays)
-#pragma unroll
-        for (int o = 32; o >= 1; o >>= 1) {
-            const float ov = __shfl_xor(bv, o, 64);
-            const int oi = __shfl_xor(bi, o, 64);
-            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-        }
-        const float sc = bv / den;
-        chosen += sc;
-        if (lane == 0) { pick_id[s] = bi; pick_sc[s] = sc; }
+        float bv;
+        int bi;
+        wave_argmax4(v, lane, bv, bi);
+        const float sc1 = bv / den;
+        chosen += sc1;
+        if (lane == 0) { pick_id[s] = bi; pick_sc[s] = sc1; }
         if ((bi & 63) == lane) v[bi >> 6] = -2.0f;
     }
-    const float inv = 1.0f / (chosen + 1e-20f);
-    for (int s = lane; s < top; s += 64) { ids[t * top + s] = pick_id[s]; wts[t * top + s] = pick_sc[s] * inv; }   // (same wave wrote them: in order)
+    const float mul = (f.renorm ? 1.0f / (chosen + 1e-20f) : 1.0f) * f.scale;
+    for (int s = lane; s < top; s += 64) { ids[t * top + s] = pick_id[s]; wts[t * top + s] = pick_sc[s] * mul; }   // (same wave wrote them: in order)
 }
 
 // Stable counting sort of the pairs by expert, one workgroup of 1024: the pairs are cut into S = 1024 / E' contiguous segments (E' = E rounded up to a
@@ -128,15 +189,16 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(int* offsets, 
     }
 }
 
-__global__ void clipped_glu_kernel(float* a, const float* gu, int ff, float limit, float alpha) {
+__global__ void clipped_glu_kernel(float* a, const float* gu, int ff, float limit, float alpha, float up_offset) {
     const long long r = blockIdx.y;
     const int f = blockIdx.x * blockDim.x + threadIdx.x;
     if (f >= ff) return;
     const float g = fminf(gu[r * 2 * ff + f], limit);
     const float u = fminf(fmaxf(gu[r * 2 * ff + ff + f], -limit), limit);
-    a[r * ff + f] = g * (1.0f / (1.0f + expf(-alpha * g))) * (u + 1.0f);
+    a[r * ff + f] = g * (1.0f / (1.0f + expf(-alpha * g))) * (u + up_offset);
 }
 
+template <bool ADD>
 __global__ void moe_combine_kernel(float* x, const float* mix, const float* d, const int* where, const float* wts, const float* shared, const float* sgate,
                                    int top, int n) {
     const long long t = blockIdx.y;
@@ -144,9 +206,9 @@ __global__ void moe_combine_kernel(float* x, const float* mix, const float* d, c
     if (i >= n) return;
     float s = 0.0f;
     for (int k = 0; k < top; ++k) s = fmaf(wts[t * top + k], d[(long long)where[t * top + k] * n + i], s);
-    if (shared) s = fmaf(sgate[t], shared[t * n + i], s);
+    if (shared) s = sgate ? fmaf(sgate[t], shared[t * n + i], s) : s + shared[t * n + i];
     if (mix) s += mix[t * n + i];
-    x[t * n + i] += s;
+    if constexpr (ADD) x[t * n + i] += s; else x[t * n + i] = s;
 }
 
 }  // namespace ntk
@@ -155,11 +217,21 @@ using namespace ntk;
 
 int ntk_moe_route(int* ids, float* wts, float* sgate, const float* h, int ldh, const float* w_router, const float* shared_gate_w, int T, int n, int E, int top,
                   void* stream) {
-    if (!ids || !wts || !h || !w_router) return NTK_E_NULL;
+    const ntk_route_desc r{0, 1, 1, 1, 1, 1.0f};   // softmax scores, no groups, weights renormalised over the chosen
+    return ntk_moe_route_ex(ids, wts, sgate, h, ldh, w_router, shared_gate_w, T, n, E, top, &r, stream);
+}
+
+int ntk_moe_route_ex(int* ids, float* wts, float* sgate, const float* h, int ldh, const float* w_router, const float* shared_gate_w, int T, int n, int E, int top,
+                     const ntk_route_desc* r, void* stream) {
+    if (!ids || !wts || !h || !w_router || !r) return NTK_E_NULL;
     if (T < 0 || n <= 0 || E <= 0 || E > kMaxExperts || top <= 0 || top > E || ldh < n) return NTK_E_SHAPE;
+    if (r->score != 0 && r->score != 1) return NTK_E_SHAPE;
+    const int groups = r->groups > 1 ? r->groups : 1;
+    if (groups > 1 && (E % groups || r->keep < 1 || r->keep > groups || r->group_top < 1 || r->group_top > 8 || (long long)r->keep * (E / groups) < top)) return NTK_E_SHAPE;
     if (T == 0) return NTK_OK;
     if ((size_t)n * 4 > 128 * 1024) return NTK_E_SHAPE;
-    hipLaunchKernelGGL(moe_route_kernel, dim3(T), dim3(kRouteThreads), (size_t)n * 4, resolve_stream(stream), ids, wts, sgate, h, ldh, w_router, shared_gate_w, n, E, top);
+    const RouteForm f{r->score, groups, r->keep, r->group_top, r->renorm, r->scale};
+    hipLaunchKernelGGL(moe_route_kernel, dim3(T), dim3(kRouteThreads), (size_t)n * 4, resolve_stream(stream), ids, wts, sgate, h, ldh, w_router, shared_gate_w, n, E, top, f);
     return last_launch_status();
 }
 
@@ -173,10 +245,14 @@ int ntk_moe_group(int* offsets, int* order, int* where, const int* ids, int T, i
 }
 
 int ntk_clipped_glu(float* a, const float* gu, int rows, int ff, float limit, float alpha, void* stream) {
+    return ntk_glu(a, gu, rows, ff, limit, alpha, 1.0f, stream);
+}
+
+int ntk_glu(float* a, const float* gu, int rows, int ff, float limit, float alpha, float up_offset, void* stream) {
     if (!a || !gu) return NTK_E_NULL;
     if (rows < 0 || ff <= 0) return NTK_E_SHAPE;
     if (rows == 0) return NTK_OK;
-    hipLaunchKernelGGL(clipped_glu_kernel, dim3((ff + 255) / 256, rows), dim3(256), 0, resolve_stream(stream), a, gu, ff, limit, alpha);
+    hipLaunchKernelGGL(clipped_glu_kernel, dim3((ff + 255) / 256, rows), dim3(256), 0, resolve_stream(stream), a, gu, ff, limit, alpha, up_offset);
     return last_launch_status();
 }
 
@@ -185,6 +261,14 @@ int ntk_moe_combine(float* x, const float* mix, const float* d, const int* where
     if (!x || !d || !where || !wts || (shared && !sgate)) return NTK_E_NULL;
     if (T < 0 || top <= 0 || n <= 0) return NTK_E_SHAPE;
     if (T == 0) return NTK_OK;
-    hipLaunchKernelGGL(moe_combine_kernel, dim3((n + 255) / 256, T), dim3(256), 0, resolve_stream(stream), x, mix, d, where, wts, shared, sgate, top, n);
+    hipLaunchKernelGGL(moe_combine_kernel<true>, dim3((n + 255) / 256, T), dim3(256), 0, resolve_stream(stream), x, mix, d, where, wts, shared, sgate, top, n);
+    return last_launch_status();
+}
+
+int ntk_moe_sum(float* out, const float* d, const int* where, const float* wts, const float* shared, const float* sgate, int T, int top, int n, void* stream) {
+    if (!out || !d || !where || !wts) return NTK_E_NULL;
+    if (T < 0 || top <= 0 || n <= 0) return NTK_E_SHAPE;
+    if (T == 0) return NTK_OK;
+    hipLaunchKernelGGL(moe_combine_kernel<false>, dim3((n + 255) / 256, T), dim3(256), 0, resolve_stream(stream), out, (const float*)nullptr, d, where, wts, shared, sgate, top, n);
     return last_launch_status();
 }

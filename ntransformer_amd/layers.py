@@ -19,7 +19,7 @@ class DenseDesc(C.Structure):
     _fields_ = [("Y", C.c_void_p), ("ldy", C.c_int), ("X", C.c_void_p), ("ldx", C.c_int), ("W", C.c_void_p), ("wstride", C.c_longlong), ("wdtype", C.c_int),
                 ("offsets", C.c_void_p), ("G", C.c_int), ("rows", C.c_void_p), ("row_div", C.c_int), ("T", C.c_int), ("N", C.c_int), ("K", C.c_int),
                 ("accumulate", C.c_int), ("glu_ff", C.c_int), ("glu_limit", C.c_float), ("glu_alpha", C.c_float),
-                ("norm_w", C.c_void_p), ("norm_eps", C.c_float), ("norm_offset", C.c_float)]
+                ("norm_w", C.c_void_p), ("norm_eps", C.c_float), ("norm_offset", C.c_float), ("glu_up_offset", C.c_float)]
 
 
 class Rotary(C.Structure):
@@ -82,7 +82,7 @@ def _i(a) -> DeviceBuffer:
 
 def dense(x: np.ndarray, w: np.ndarray, dtype: str = "float32", offsets=None, rows=None, row_div: int = 1, n_rows: Optional[int] = None,
           y0: Optional[np.ndarray] = None, glu_limit: Optional[float] = None, glu_alpha: float = 1.702, norm_w: Optional[np.ndarray] = None,
-          norm_eps: float = 1e-6, norm_offset: float = 0.0) -> np.ndarray:
+          norm_eps: float = 1e-6, norm_offset: float = 0.0, glu_up_offset: float = 1.0) -> np.ndarray:
     """y[r] = x[src(r)] . w[g(r)]^T; w [N, K] or a stack [G, N, K] with `offsets` [G + 1]; rows: source row per output row (divided by row_div);
     y0: start values to accumulate onto."""
     L = _bind()
@@ -95,7 +95,7 @@ def dense(x: np.ndarray, w: np.ndarray, dtype: str = "float32", offsets=None, ro
     ob = _i(offsets) if offsets is not None else None
     rb = _i(rows) if rows is not None else None
     d = DenseDesc(yb.ptr, N, xb.ptr, x.shape[1], wb.ptr, N * K if stacked else 0, wdt, ob.ptr if ob else None, w.shape[0] if stacked else 1,
-                  rb.ptr if rb else None, row_div, T, N, K, int(y0 is not None), 0, 0.0, 0.0, None, 0.0, 0.0)
+                  rb.ptr if rb else None, row_div, T, N, K, int(y0 is not None), 0, 0.0, 0.0, None, 0.0, 0.0, glu_up_offset)
     nb = _f(norm_w) if norm_w is not None else None
     if nb is not None:          # fused RMS norm of the activation rows (few rows)
         d.norm_w, d.norm_eps, d.norm_offset = nb.ptr, norm_eps, norm_offset
