@@ -26,6 +26,16 @@ class Rotary(C.Structure):
     _fields_ = [("freq", C.c_void_p), ("mag", C.c_float), ("dims", C.c_int)]
 
 
+class WindowAttentionDesc(C.Structure):
+    _fields_ = [("out", C.c_void_p), ("ldo", C.c_int), ("q", C.c_void_p), ("ldq", C.c_int), ("cache", C.c_void_p), ("row", C.c_int),
+                ("H", C.c_int), ("G", C.c_int), ("maps", C.c_int), ("dn", C.c_int), ("dv", C.c_int), ("pos0", C.c_int), ("T", C.c_int), ("window", C.c_int),
+                ("scale", C.c_float), ("lam", C.c_float), ("sub_norm", C.c_int), ("eps", C.c_float), ("out_scale", C.c_float), ("scratch", C.c_void_p)]
+
+
+class RouteDesc(C.Structure):
+    _fields_ = [("score", C.c_int), ("groups", C.c_int), ("keep", C.c_int), ("group_top", C.c_int), ("renorm", C.c_int), ("scale", C.c_float)]
+
+
 def _bind():
     L = _lib.lib()
     if getattr(L, "_layers_bound", False):
@@ -49,6 +59,21 @@ def _bind():
     L.ntk_moe_group.argtypes = [vp, vp, vp, vp, i, i, i, vp]
     L.ntk_clipped_glu.argtypes = [vp, vp, i, i, f, f, vp]
     L.ntk_moe_combine.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, vp]
+    L.ntk_embed_dense_scaled.argtypes = [vp, vp, i, vp, i, i, i, f, vp]
+    L.ntk_scale.argtypes = [vp, ll, f, vp]
+    L.ntk_layernorm.argtypes = [vp, i, vp, i, vp, vp, i, i, f, i, vp]
+    L.ntk_layernorm_history.argtypes = [vp, vp, i, vp, vp, vp, i, i, i, i, f, vp]
+    L.ntk_causal_conv_mix.argtypes = [vp, i, vp, vp, vp, i, i, i, vp]
+    L.ntk_polynorm.argtypes = [vp, i, vp, i, vp, i, i, f, vp]
+    L.ntk_gated_rmsnorm.argtypes = [vp, i, vp, i, vp, vp, i, i, i, f, vp]
+    L.ntk_window_prepare.argtypes = [vp, i, vp, i, vp, i, vp, i, i, i, i, i, i, C.POINTER(Rotary), i, i, vp]
+    L.ntk_window_attention_scratch.argtypes = [i, i, i, i, i]
+    L.ntk_window_attention_scratch.restype = C.c_size_t
+    L.ntk_window_attention.argtypes = [C.POINTER(WindowAttentionDesc), vp]
+    L.ntk_lightning_attention.argtypes = [vp, i, vp, i, vp, i, vp, i, vp, vp, i, i, i, i, i, i, vp]
+    L.ntk_moe_route_ex.argtypes = [vp, vp, vp, vp, i, vp, vp, i, i, i, i, C.POINTER(RouteDesc), vp]
+    L.ntk_glu.argtypes = [vp, vp, i, i, f, f, f, vp]
+    L.ntk_moe_sum.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, vp]
     L._layers_bound = True
     return L
 
@@ -215,3 +240,122 @@ def moe_combine(x, mix, d, where, wts, shared=None, sgate=None) -> np.ndarray:
     gb = _f(sgate) if sgate is not None else None
     check(L.ntk_moe_combine(xb.ptr, mb.ptr if mb else None, db.ptr, wb.ptr, tb.ptr, sb.ptr if sb else None, gb.ptr if gb else None, T, top, n, None), "ntk_moe_combine")
     return xb.numpy(np.float32, T * n).reshape(T, n)
+
+
+# ---------------------------------------------------------------------------------------------------------------- sequential-form operators
+def layernorm(x: np.ndarray, w: np.ndarray, b: Optional[np.ndarray], eps: float, onto: Optional[np.ndarray] = None) -> np.ndarray:
+    """(x - mean) / sqrt(var + eps) * w + b per row; onto: start values the result is added to"""
+    L = _bind()
+    T, n = x.shape
+    xb, wb = _f(x), _f(w)
+    bb = _f(b) if b is not None else None
+    yb = _f(onto) if onto is not None else DeviceBuffer.zeros(T * n * 4)
+    check(L.ntk_layernorm(yb.ptr, n, xb.ptr, n, wb.ptr, bb.ptr if bb else None, T, n, eps, int(onto is not None), None), "ntk_layernorm")
+    return yb.numpy(np.float32, T * n).reshape(T, n)
+
+
+def norm_conv(x: np.ndarray, w: np.ndarray, b: np.ndarray, eps: float, canon: np.ndarray, state: Optional[np.ndarray], pos0: int):
+    """h = layer norm of x; -> (h + causal convolution of h with the carried inputs in front, the new carried inputs [taps - 1, n])"""
+    L = _bind()
+    T, n = x.shape
+    taps = canon.shape[1]
+    xb, wb, bb, cb = _f(x), _f(w), _f(b), _f(canon)
+    sb = _f(state) if state is not None else DeviceBuffer.zeros(max(taps - 1, 1) * n * 4)
+    hist, out = DeviceBuffer.zeros((T + taps - 1) * n * 4), DeviceBuffer.zeros(T * n * 4)
+    check(L.ntk_layernorm_history(hist.ptr, xb.ptr, n, wb.ptr, bb.ptr, sb.ptr, taps, pos0, T, n, eps, None), "ntk_layernorm_history")
+    check(L.ntk_causal_conv_mix(out.ptr, n, hist.ptr, cb.ptr, sb.ptr, taps, T, n, None), "ntk_causal_conv_mix")
+    return out.numpy(np.float32, T * n).reshape(T, n), sb.numpy(np.float32, max(taps - 1, 1) * n).reshape(-1, n)[:taps - 1]
+
+
+def polynorm(z: np.ndarray, coef, eps: float) -> np.ndarray:
+    L = _bind()
+    T, n = z.shape
+    zb, cb = _f(z), _f(np.asarray(coef, np.float32))
+    out = DeviceBuffer.zeros(T * n * 4)
+    check(L.ntk_polynorm(out.ptr, n, zb.ptr, n, cb.ptr, T, n, eps, None), "ntk_polynorm")
+    return out.numpy(np.float32, T * n).reshape(T, n)
+
+
+def gated_rmsnorm(x: np.ndarray, w: np.ndarray, g: Optional[np.ndarray], eps: float) -> np.ndarray:
+    L = _bind()
+    T, n = x.shape
+    xb, wb = _f(x), _f(w)
+    gb = _f(g) if g is not None else None
+    out = DeviceBuffer.zeros(T * n * 4)
+    check(L.ntk_gated_rmsnorm(out.ptr, n, xb.ptr, n, wb.ptr, gb.ptr if gb else None, n, T, n, eps, None), "ntk_gated_rmsnorm")
+    return out.numpy(np.float32, T * n).reshape(T, n)
+
+
+def window_prepare(q: np.ndarray, k: np.ndarray, v: np.ndarray, H: int, G: int, maps: int, dn: int, dv: int, freq: np.ndarray, dims: int, pos0: int,
+                   cache: Optional[np.ndarray] = None, cache_rows: Optional[int] = None):
+    """-> (cache [rows, G * (maps * dn + dv)] with rows pos0 .. filled, q rotated)"""
+    L = _bind()
+    T, row = q.shape[0], G * (maps * dn + dv)
+    n = cache_rows or (pos0 + T)
+    cb = _f(cache) if cache is not None else DeviceBuffer.zeros(n * row * 4)
+    qb, kb, vb = _f(q), _f(k), _f(v)
+    fb = DeviceBuffer.from_numpy(np.ascontiguousarray(freq if len(freq) else [0.0], np.float64))
+    rot = Rotary(fb.ptr, 1.0, dims)
+    check(L.ntk_window_prepare(cb.ptr, row, qb.ptr, q.shape[1], kb.ptr, k.shape[1], vb.ptr, v.shape[1], H, G, maps, dn, dv, C.byref(rot), pos0, T, None), "ntk_window_prepare")
+    return cb.numpy(np.float32, n * row).reshape(n, row), qb.numpy(np.float32, q.size).reshape(q.shape)
+
+
+def window_attention(q: np.ndarray, cache: np.ndarray, H: int, G: int, maps: int, dn: int, dv: int, pos0: int, window: int, scale: float, lam: float = 0.0,
+                     sub_norm: bool = False, eps: float = 1e-6, out_scale: float = 1.0, split: bool = True) -> np.ndarray:
+    """q [T, H * maps * dn] (rotated), cache rows [G][maps][dn] keys | [G][dv] values; split: long key ranges of few rows may be cut into merged parts"""
+    L = _bind()
+    T, row = q.shape[0], G * (maps * dn + dv)
+    qb, cb = _f(q), _f(cache)
+    out = DeviceBuffer.zeros(T * H * dv * 4)
+    sc = DeviceBuffer.zeros(max(int(L.ntk_window_attention_scratch(T, H, maps, dv, pos0 + T)), 1) * 4) if split else None
+    d = WindowAttentionDesc(out.ptr, H * dv, qb.ptr, q.shape[1], cb.ptr, row, H, G, maps, dn, dv, pos0, T, window, scale, lam, int(sub_norm), eps, out_scale,
+                            sc.ptr if sc else None)
+    check(L.ntk_window_attention(C.byref(d), None), "ntk_window_attention")
+    return out.numpy(np.float32, T * H * dv).reshape(T, H * dv)
+
+
+def lightning_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, decay, H: int, dn: int, dv: int, pos0: int, state: Optional[np.ndarray] = None, silu: bool = True):
+    """-> (out [T, H * dv], state [H, dn, dv]); state: what an earlier portion left (ignored when pos0 == 0)"""
+    L = _bind()
+    T = q.shape[0]
+    qb, kb, vb = _f(q), _f(k), _f(v)
+    with np.errstate(divide="ignore"):
+        lb = _f(np.log(np.asarray(decay, np.float64)))
+    sb = _f(state) if state is not None else DeviceBuffer.from_numpy(np.full(H * dn * dv, np.nan, np.float32))
+    out = DeviceBuffer.zeros(T * H * dv * 4)
+    check(L.ntk_lightning_attention(out.ptr, H * dv, qb.ptr, q.shape[1], kb.ptr, k.shape[1], vb.ptr, v.shape[1], lb.ptr, sb.ptr, H, dn, dv, int(silu), pos0, T, None),
+          "ntk_lightning_attention")
+    return out.numpy(np.float32, T * H * dv).reshape(T, H * dv), sb.numpy(np.float32, H * dn * dv).reshape(H, dn, dv)
+
+
+def moe_route_ex(h: np.ndarray, w_router: np.ndarray, top: int, score: int = 1, groups: int = 1, keep: int = 1, group_top: int = 2, renorm: bool = False,
+                 scale: float = 1.0):
+    L = _bind()
+    T, n = h.shape
+    E = w_router.shape[0]
+    hb, wb = _f(h), _f(w_router)
+    ids, wts = DeviceBuffer.zeros(T * top * 4), DeviceBuffer.zeros(T * top * 4)
+    r = RouteDesc(score, groups, keep, group_top, int(renorm), scale)
+    check(L.ntk_moe_route_ex(ids.ptr, wts.ptr, None, hb.ptr, n, wb.ptr, None, T, n, E, top, C.byref(r), None), "ntk_moe_route_ex")
+    return ids.numpy(np.int32, T * top).reshape(T, top), wts.numpy(np.float32, T * top).reshape(T, top)
+
+
+def glu(gu: np.ndarray, limit: float = float("inf"), alpha: float = 1.0, up_offset: float = 0.0) -> np.ndarray:
+    L = _bind()
+    rows, ff = gu.shape[0], gu.shape[1] // 2
+    gb = _f(gu)
+    out = DeviceBuffer.zeros(rows * ff * 4)
+    check(L.ntk_glu(out.ptr, gb.ptr, rows, ff, limit, alpha, up_offset, None), "ntk_glu")
+    return out.numpy(np.float32, rows * ff).reshape(rows, ff)
+
+
+def moe_sum(d, where, wts, shared=None, sgate=None) -> np.ndarray:
+    L = _bind()
+    T, top = wts.shape
+    n = d.shape[1]
+    db, wb, tb = _f(d), _i(where), _f(wts)
+    sb = _f(shared) if shared is not None else None
+    gb = _f(sgate) if sgate is not None else None
+    out = DeviceBuffer.zeros(T * n * 4)
+    check(L.ntk_moe_sum(out.ptr, db.ptr, wb.ptr, tb.ptr, sb.ptr if sb else None, gb.ptr if gb else None, T, top, n, None), "ntk_moe_sum")
+    return out.numpy(np.float32, T * n).reshape(T, n)

@@ -226,6 +226,44 @@ def forward(cfg, w, tokens, return_layers=False):
     return (logits, torch.stack(streams)) if return_layers else logits
 
 
+def closest_call(cfg, w, tokens):
+    """The smallest gap, over all positions and mixture layers, between a score (or group score) that was taken and the best one that was not:
+    a model and tokens whose gap is wide give the same choice of experts under bfloat16 rounding."""
+    eps = cfg["norm"]["eps"]
+    x = w["embed"][torch.tensor(list(tokens))] * cfg["embedding"]["scale"]
+    gap = math.inf
+    for i in layer_runs(cfg):
+        L, p = cfg["layers"][i], "l%d." % i
+        h, _ = conv_added(layer_norm(x, w[p + "norm1"], w[p + "norm1.b"], eps), w[p + "canon1"])
+        y = diff_attention(h, w, p + "mix.", L["mixer"], eps)[0] if L["type"] == "attention" else lightning(h, w, p + "mix.", L["mixer"], eps)[0]
+        x = x + layer_norm(y, w[p + "norm1b"], w[p + "norm1b.b"], eps)
+        ml = L.get("mlp")
+        if not ml:
+            continue
+        h, _ = conv_added(layer_norm(x, w[p + "norm2"], w[p + "norm2.b"], eps), w[p + "canon2"])
+        if ml["kind"] == "moe":
+            rt = ml["router"]
+            s = torch.sigmoid(h @ w[p + "mlp.router"].T)
+            E, gr = s.shape[1], rt.get("groups")
+            for t in range(s.shape[0]):
+                allowed = torch.ones(E, dtype=torch.bool)
+                if gr and gr["count"] > 1:
+                    per = E // gr["count"]
+                    gs = torch.sort(torch.stack([torch.sort(s[t, g * per:(g + 1) * per], descending=True).values[:2].sum() for g in range(gr["count"])]),
+                                    descending=True)
+                    if gr["keep"] < gr["count"]:
+                        gap = min(gap, float(gs.values[gr["keep"] - 1] - gs.values[gr["keep"]]))
+                    allowed[:] = False
+                    for g in gs.indices[:gr["keep"]].tolist():
+                        allowed[g * per:(g + 1) * per] = True
+                sc = torch.sort(s[t][allowed], descending=True).values
+                if rt["top"] < sc.numel():
+                    gap = min(gap, float(sc[rt["top"] - 1] - sc[rt["top"]]))
+        y = dense_ff(h, w, p + "mlp.", eps) if ml["kind"] == "dense" else mixture(h, w, p + "mlp.", ml)
+        x = x + layer_norm(y, w[p + "norm2b"], w[p + "norm2b.b"], eps)
+    return gap
+
+
 def greedy(cfg, w, prompt, n):
     toks = list(prompt)
     for _ in range(n):
