@@ -60,11 +60,11 @@ def parse():
     ap.add_argument("--cpu-tokens", type=int, default=128, help="-n of the reference CLI run that is the CPU baseline (BASELINE config 1: 128)")
     ap.add_argument("--no-also", action="store_true", help="skip the other BASELINE configurations (8B Q4_K_M, 70B Q4_K_M, 70B Q6_K, 8B Q8_0 behind 3900- and 32768-token prompts)")
     ap.add_argument("--no-pmc-note", action="store_true")
-    ap.add_argument("--family", default="", choices=["", "fabolorn"],
-                    help="instead of the default workload: prompt and decode throughput of a layer-list family on synthetic real-sized layers, beside the "
-                         "Llama path at equal width / heads / active feed-forward width (F16 and Q8_0); one JSON line of its own")
+    ap.add_argument("--family", default="", choices=["", "fabolorn", "nizorax"],
+                    help="instead of the default workload: prompt and decode throughput of a layer-list family on synthetic real-sized layers; beside it, fabolorn: the "
+                         "Llama path at equal width / heads / active feed-forward width (F16 and Q8_0), nizorax: the fabolorn family at the same preset; one JSON line of its own")
     ap.add_argument("--family-size", default="lite", choices=["tiny", "lite", "mid"])
-    ap.add_argument("--family-no-compare", action="store_true", help="skip the Llama runs beside the family (a profile of the family's kernels alone)")
+    ap.add_argument("--family-no-compare", action="store_true", help="skip the runs beside the family (a profile of the family's kernels alone)")
     ap.add_argument("--family-layers", type=int, default=2)
     ap.add_argument("--family-dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prompt-bench", type=int, default=1024, help="also time one prompt pass of this many tokens (0 = skip); reported under config.prompt_pass")
@@ -389,24 +389,14 @@ def roofline_block(args, model, mix, r):
             "token_ms_by_class_eager": {"gemv": round(r["ms"][0], 4), "attention": round(r["ms"][1], 4), "other": round(r["ms"][2], 4)}}
 
 
-def run_family(args):
-    """--family fabolorn: a synthetic model folder of `--family-layers` real-sized layers (ntransformer_amd/synth_folder.py), a prompt pass of
-    --prompt-bench tokens (second of two runs) and --steps decoded tokens behind it through the slot cache; then the Llama path with the same width,
-    heads (head size 128), layers, vocabulary and ACTIVE feed-forward width (top x ff + shared ff) as F16 and as Q8_0, same prompt and decode."""
+def time_folder(args, cfg, prompt, ctx):
+    """prompt pass (second of two runs) and --steps decoded tokens behind it, through the slot cache of a synthetic model folder"""
     import shutil
     import tempfile
-    import numpy as np
-    from ntransformer_amd import _lib, synth_folder
+    from ntransformer_amd import synth_folder
     from ntransformer_amd import engine as E
-    L = _lib.lib()
-    _lib.check(L.ntk_device_init(0), "ntk_device_init")
-    cfg = synth_folder.fabolorn_config(args.family_size, args.family_layers)
-    p = synth_folder.PRESETS[args.family_size]
-    T, ctx = args.prompt_bench or 1024, max(args.ctx, (args.prompt_bench or 1024) + args.steps + args.warmup + 8)
+    T = len(prompt)
     tmp = tempfile.mkdtemp(prefix="ntk_family_")
-    rng = np.random.Generator(np.random.Philox(key=[20260925, 7]))
-    prompt = [int(t) for t in rng.integers(0, p["vocab"], T)]
-    out = {}
     try:
         nbytes = synth_folder.write_folder(tmp, cfg)
         eng = E.Engine()
@@ -425,12 +415,36 @@ def run_family(args):
         for _ in range(args.steps):
             tok = int(eng.seq_forward(s, [tok], want=[0])[0].argmax())
         t_dec = time.perf_counter() - t0
-        out["fabolorn"] = {"prompt_tok_s": round(T / t_prompt, 1), "decode_tok_s": round(args.steps / t_dec, 1), "decode_ms_per_token": round(1e3 * t_dec / args.steps, 3),
-                           "weight_bytes": eng.weight_bytes(), "file_bytes": nbytes}
+        res = {"prompt_tok_s": round(T / t_prompt, 1), "decode_tok_s": round(args.steps / t_dec, 1), "decode_ms_per_token": round(1e3 * t_dec / args.steps, 3),
+               "weight_bytes": eng.weight_bytes(), "file_bytes": nbytes}
         eng.close()
+        return res
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
-    for mix in (() if args.family_no_compare else ("F16", "Q8_0")):
+
+
+def run_family(args):
+    """--family fabolorn | nizorax: a synthetic model folder of `--family-layers` real-sized layers (ntransformer_amd/synth_folder.py), a prompt pass of
+    --prompt-bench tokens (second of two runs) and --steps decoded tokens behind it through the slot cache.  Beside it, unless --family-no-compare:
+    fabolorn -- the Llama path with the same width, heads (head size 128), layers, vocabulary and ACTIVE feed-forward width (top x ff + shared ff) as
+    F16 and as Q8_0, same prompt and decode; nizorax -- the Fabolorn family (the closest model: same layer stack, slots and products) at the same preset."""
+    import numpy as np
+    from ntransformer_amd import _lib, synth_folder
+    from ntransformer_amd import engine as E
+    L = _lib.lib()
+    _lib.check(L.ntk_device_init(0), "ntk_device_init")
+    p = synth_folder.PRESETS[args.family_size]
+    T, ctx = args.prompt_bench or 1024, max(args.ctx, (args.prompt_bench or 1024) + args.steps + args.warmup + 8)
+    rng = np.random.Generator(np.random.Philox(key=[20260925, 7]))
+    prompt = [int(t) for t in rng.integers(0, p["vocab"], T)]
+    out = {}
+    if args.family == "nizorax":
+        out["nizorax"] = time_folder(args, synth_folder.nizorax_config(args.family_size, args.family_layers), prompt, ctx)
+        if not args.family_no_compare:
+            out["fabolorn"] = time_folder(args, synth_folder.fabolorn_config(args.family_size, args.family_layers), prompt, ctx)
+    else:
+        out["fabolorn"] = time_folder(args, synth_folder.fabolorn_config(args.family_size, args.family_layers), prompt, ctx)
+    for mix in (() if args.family_no_compare or args.family != "fabolorn" else ("F16", "Q8_0")):
         try:
             inter = p["top"] * p["ff"] + p["shared_ff"]
             inter -= inter % 256
@@ -451,9 +465,10 @@ def run_family(args):
             eng.close()
         except Exception as e:
             out["llama_" + mix.lower()] = {"error": repr(e)}
-    print(json.dumps({"metric": "fabolorn_decode_tokens_per_s", "value": out["fabolorn"]["decode_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
-                      "warmup": args.warmup, "ms_per_step": out["fabolorn"]["decode_ms_per_token"], "higher_is_better": True, "dtype": args.family_dtype,
-                      "data": "synthetic", "config": {"family": "fabolorn", "size": args.family_size, "layers": args.family_layers, "prompt_tokens": T,
+    fam = args.family
+    print(json.dumps({"metric": fam + "_decode_tokens_per_s", "value": out[fam]["decode_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+                      "warmup": args.warmup, "ms_per_step": out[fam]["decode_ms_per_token"], "higher_is_better": True, "dtype": args.family_dtype,
+                      "data": "synthetic", "config": {"family": fam, "size": args.family_size, "layers": args.family_layers, "prompt_tokens": T,
                                                       "preset": p}, "results": out}))
 
 

@@ -68,6 +68,70 @@ def fabolorn_shapes(cfg: dict) -> Dict[str, Tuple[int, ...]]:
     return s
 
 
+def nizorax_config(preset: str, layers: int = 2) -> dict:
+    """the sequential family at the preset's width, heads, experts and vocabulary: attention layers (two score maps of half the preset's key size each,
+    four query heads per key/value head, the preset's window) alternate with lightning layers; every third layer has the dense feed-forward at the
+    mixture's active width, the others the mixture (groups of eight experts, half of the groups open)"""
+    p = PRESETS[preset]
+    H, dn = p["heads"], p["dim"] + p["rot_dim"]
+    ls = []
+    for k in range(layers):
+        if k % 2 == 0:
+            mx = {"heads": H, "kv_heads": max(H // 4, 1), "dim": dn // 2, "vdim": p["vdim"], "diff": 0.8, "scale": 1.0 / math.sqrt(dn // 2),
+                  "mask": {"size": p["window"]}, "rot": {"base": 1000000.0, "dims": dn // 4, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 4096}}}
+            t = "attention"
+        else:
+            mx = {"heads": H, "dim": dn // 2 if dn // 2 <= 128 else 128, "vdim": p["vdim"], "decay": [1.0 - 2.0 ** (-5.0 - 3.0 * h / max(H - 1, 1)) for h in range(H)]}
+            t = "lightning"
+        if k % 3 == 2:
+            ml = {"kind": "dense", "ff": p["top"] * p["ff"] + p["shared_ff"]}
+        else:
+            per = 8 if p["experts"] % 8 == 0 and p["experts"] >= 16 else 1
+            ml = {"kind": "moe", "expert": {"ff": p["ff"]}, "router": {"experts": p["experts"], "top": p["top"], "scale": 2.0}, "shared": {"ff": p["shared_ff"]}}
+            if per > 1:
+                ml["router"]["groups"] = {"count": p["experts"] // per, "keep": max(p["experts"] // per // 2, 1)}
+        ls.append({"type": t, "mixer": mx, "mlp": ml})
+    return {"architecture": "Nizorax", "layers": ls, "norm": {"eps": 1e-5}, "canon": {"taps": 4}, "embedding": {"scale": math.sqrt(p["width"])},
+            "logit_scale": 1.0 / math.sqrt(p["width"]), "vocab": p["vocab"], "width": p["width"]}
+
+
+def nizorax_shapes(cfg: dict) -> Dict[str, Tuple[int, ...]]:
+    W, V, taps = cfg["width"], cfg["vocab"], cfg["canon"]["taps"]
+    s: Dict[str, Tuple[int, ...]] = {"embed": (V, W), "final.norm": (W,), "final.norm.b": (W,), "head": (V, W)}
+    for i, L in enumerate(cfg["layers"]):
+        p, mx, ml = "l%d." % i, L["mixer"], L.get("mlp")
+        for nm in ("norm1", "norm1b") + (("norm2", "norm2b") if ml else ()):
+            s[p + nm], s[p + nm + ".b"] = (W,), (W,)
+        s[p + "canon1"] = (W, taps)
+        if ml:
+            s[p + "canon2"] = (W, taps)
+        H, dn, dv = mx["heads"], mx["dim"], mx["vdim"]
+        if L["type"] == "attention":
+            G = mx.get("kv_heads", H)
+            s[p + "mix.q"], s[p + "mix.k"], s[p + "mix.v"], s[p + "mix.o"] = (H * 2 * dn, W), (G * 2 * dn, W), (G * dv, W), (W, H * dv)
+            for nm in ("lq1", "lk1", "lq2", "lk2"):
+                s[p + "mix." + nm] = (dn,)
+        else:
+            s[p + "mix.q"], s[p + "mix.k"], s[p + "mix.v"], s[p + "mix.g"] = (H * dn, W), (H * dn, W), (H * dv, W), (H * dv, W)
+            s[p + "mix.o"], s[p + "mix.norm"] = (W, H * dv), (H * dv,)
+        if ml and ml["kind"] == "dense":
+            s[p + "mlp.up"], s[p + "mlp.down"], s[p + "mlp.act"] = (ml["ff"], W), (W, ml["ff"]), (4,)
+        elif ml:
+            ff = ml["expert"]["ff"]
+            for e in range(ml["router"]["experts"]):
+                q = "%smlp.e%d." % (p, e)
+                s[q + "gate"], s[q + "up"], s[q + "down"] = (ff, W), (ff, W), (W, ff)
+            s[p + "mlp.router"] = (ml["router"]["experts"], W)
+            if ml.get("shared"):
+                sf = ml["shared"]["ff"]
+                s[p + "mlp.shared.gate"], s[p + "mlp.shared.up"], s[p + "mlp.shared.down"] = (sf, W), (sf, W), (W, sf)
+    return s
+
+
+def shapes_of(cfg: dict) -> Dict[str, Tuple[int, ...]]:
+    return nizorax_shapes(cfg) if cfg.get("architecture") == "Nizorax" else fabolorn_shapes(cfg)
+
+
 def _bf16(a: np.ndarray) -> np.ndarray:
     u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
     return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
@@ -78,7 +142,7 @@ def write_folder(folder: str, cfg: dict, seed: int = 20260925) -> int:
     os.makedirs(folder, exist_ok=True)
     with open(os.path.join(folder, "config.json"), "w") as f:
         json.dump(cfg, f)
-    shapes = fabolorn_shapes(cfg)
+    shapes = shapes_of(cfg)
     g = np.random.default_rng(seed)
     pool = g.standard_normal(1 << 22).astype(np.float32)
     header, at = {}, 0
@@ -94,7 +158,10 @@ def write_folder(folder: str, cfg: dict, seed: int = 20260925) -> int:
         for k, (name, shp) in enumerate(shapes.items()):
             n = int(np.prod(shp))
             if len(shp) == 1:
-                vals = 0.1 * pool[:n] + (1.0 if name.endswith(".norm") and name != "final.norm" else 0.0)
+                around_one = name.endswith(".norm") and name != "final.norm"
+                if cfg.get("architecture") == "Nizorax":     # layer-norm weights around one, biases / lambda vectors / activation numbers small
+                    around_one = name.rsplit(".", 1)[-1] in ("norm", "norm1", "norm2", "norm1b", "norm2b")
+                vals = 0.1 * pool[:n] + (1.0 if around_one else 0.0)
                 f.write(_bf16(vals).tobytes())
                 continue
             scale = 1.0 if name == "embed" else 1.0 / math.sqrt(shp[-1])
