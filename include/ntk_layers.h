@@ -80,6 +80,13 @@ int ntk_layernorm(float* y, int ldy, const float* x, int ldx, const float* w, co
 int ntk_layernorm_history(float* hist, const float* x, int ldx, const float* w, const float* b, const float* state, int taps, int pos0, int T, int n, float eps,
                           void* stream);
 int ntk_causal_conv_mix(float* out, int ldo, const float* hist, const float* w, float* state, int taps, int T, int n, void* stream);
+/* The whole seam between two sublayers of a layer whose sublayer outputs are normed before they join the stream, in one call:
+ *   x[t] += layer norm of add_y[t] with (add_w, add_b)     -- the output still owed to the stream; add_y == NULL: nothing is owed
+ *   h[t]  = layer norm of x[t] with (w, b);  out[t] = h[t] + conv(h)[t] as above, `state` carried on.
+ * One token runs as ONE launch (the history of a channel belongs to the thread that owns it); more tokens as ntk_layernorm_history's kernel with the owed
+ * output folded in, then ntk_causal_conv_mix (hist: [(taps - 1) + T][n] floats of work space, unused for T == 1).  Same sums in the same order either way. */
+int ntk_sandwich_norm_conv(float* out, int ldo, float* x, int ldx, const float* add_y, int ldy, const float* add_w, const float* add_b, const float* w, const float* b,
+                           const float* canon, float* state, float* hist, int taps, int pos0, int T, int n, float eps, void* stream);
 /* y[t][i] = a N(z)_i + b N(z^2)_i + c N(z^3)_i + e with (a, b, c, e) = coef[0..3] (device F32), powers element by element and
  * N(u) = u / sqrt(mean(u^2) + eps) over the row of n values */
 int ntk_polynorm(float* y, int ldy, const float* z, int ldz, const float* coef, int T, int n, float eps, void* stream);
@@ -146,9 +153,12 @@ int ntk_window_attention(const ntk_window_attention_desc* d, void* stream);
  * Linear attention with a per-head decay: S_t = decay_h S_(t-1) + k_t v_t^T (S [dn][dv] per head, F32), o_t = S_t^T q_t, with q, k, v = act(raw)
  * (act = silu when silu != 0) applied on the way in.  Portions are walked in chunks (scores inside a chunk, the state between chunks), all in F32.
  * q [T][H][dn], k [T][H][dn], v [T][H][dv] with ldq / ldk / ldv floats between tokens; log_decay device F32 [H] = ln(decay_h) (-inf for 0);
- * state [H][dn][dv]: read unless pos0 == 0 (a sequence starts from zeros), written at the end.  out [T][H][dv].  dn <= 256. */
+ * state [H][dn][dv]: read unless pos0 == 0 (a sequence starts from zeros), written at the end.  out [T][H][dv].  dn <= 256.
+ * scratch: F32 [>= ntk_lightning_attention_scratch(...)] lets the chunks of a long portion run side by side (three launches); NULL: one workgroup per
+ * (head, 64 value columns) walks them in turn.  Up to 8 tokens (decoding) take a form of their own that keeps the state in registers. */
+size_t ntk_lightning_attention_scratch(int T, int H, int dn, int dv);
 int ntk_lightning_attention(float* out, int ldo, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* log_decay, float* state,
-                            int H, int dn, int dv, int silu, int pos0, int T, void* stream);
+                            int H, int dn, int dv, int silu, int pos0, int T, float* scratch, void* stream);
 
 /* ---- moe.hip ---------------------------------------------------------------------------------------------------------------------- */
 /* Router of a mixture of experts, one launch: z = W_r h (F32 weights [E][n]), s = softmax(z); the `top` largest (ties: the lower index), weights

@@ -447,6 +447,10 @@ int LayerStackModel::load(const std::string& dir, const SeqLoadOptions& opt) {
     LS_TRY(upload_matrix(f, {"head"}, W, head_));
     if (embed_.out_f != info_.vocab || head_.out_f != info_.vocab) return fail(NTK_E_SHAPE, "embed / head do not have 'vocab' rows");
     LS_TRY(upload_norm(f, "final.norm", final_norm_));
+    if (final_norm_.b && logit_scale_ != 1.0f) {   // logits = head (norm x) * scale = head (norm x with weight and bias times scale): no launch of its own per step
+        if (ntk_scale(final_norm_.w, W, logit_scale_, stream_) != NTK_OK || ntk_scale(final_norm_.b, W, logit_scale_, stream_) != NTK_OK) return fail(NTK_E_LAUNCH, "scaling the output norm failed");
+        logit_scale_ = 1.0f;
+    }
     if (has_loop_ && form_.loop_projection) {
         LS_TRY(upload_matrix(f, {"loop.in"}, 2 * W, loop_in_));
         if (loop_in_.out_f != W) return fail(NTK_E_SHAPE, "tensor 'loop.in' is not [width, 2 width]");
@@ -460,7 +464,7 @@ int LayerStackModel::load(const std::string& dir, const SeqLoadOptions& opt) {
 int LayerStackModel::alloc_buffers() {
     const int W = info_.width;
     chunk_ = std::min(opt_.max_context, 1024);
-    size_t sc = 0, wsc = 0;
+    size_t sc = 0, wsc = 0, lsc = 0;
     for (const auto& L : layers_) {
         if (L.mixer == kMixLatent) {
             const LatentMixer& m = L.mix;
@@ -483,6 +487,7 @@ int LayerStackModel::alloc_buffers() {
             const LightningMixer& m = L.lin;
             max_in_ = std::max<int>(max_in_, (int)m.in.out_f);
             max_hdv_ = std::max(max_hdv_, m.heads * m.vdim);
+            lsc = std::max(lsc, ntk_lightning_attention_scratch(chunk_, m.heads, m.dim, m.vdim));
         }
         if (L.mlp_kind == kMlpMoe) {
             max_top_ = std::max(max_top_, L.mlp.top);
@@ -501,7 +506,7 @@ int LayerStackModel::alloc_buffers() {
     if (max_hqd_ > 0)      // latent mixers: query latents, folded queries, the up-projected keys and values of the visible range
         ok = ok && fl(&cat_, C * 2 * W) && fl(&cq_, C * std::max(max_qrank_, 1)) && fl(&q_, C * max_hqd_) && fl(&qf_, (size_t)kSharedRows * max_fold_) &&
              fl(&lat_, (size_t)kSharedRows * max_hr_) && fl(&kx_, ctx * max_hdn_) && fl(&vx_, ctx * max_hdv_) && fl(&scratch_, sc);
-    if (form_.sequential) ok = ok && fl(&hist_, (C + (size_t)taps_ - 1) * W) && fl(&ff_, C * W) && fl(&zf_, C * max_ffn_) && fl(&wscratch_, wsc);
+    if (form_.sequential) ok = ok && fl(&hist_, (C + (size_t)taps_ - 1) * W) && fl(&ff_, C * W) && fl(&zf_, C * max_ffn_) && fl(&wscratch_, wsc) && fl(&lscratch_, lsc);
     want_dev_ = tokens_dev_ ? tokens_dev_ + C : nullptr;   // one staging area: [tokens of a pass | wanted places], filled by ONE stream-ordered copy from pinned memory
     h_stage_ = (int*)nt_hip_malloc_host(2 * C * sizeof(int));
     ok = ok && h_stage_ != nullptr;
@@ -603,7 +608,7 @@ int LayerStackModel::run_lightning(const StackLayer& L, float* state, int T, int
     const LightningMixer& m = L.lin;
     const int W = info_.width, na = (int)m.in.out_f, hv = m.heads * m.vdim;
     LS_TRY(ntk_dense_linear(a_, na, h1_, W, m.in.ptr, m.in.dtype, T, na, W, 0, stream_));
-    LS_TRY(ntk_lightning_attention(att_, hv, a_, na, a_ + m.k_off, na, a_ + m.v_off, na, m.log_decay, state, m.heads, m.dim, m.vdim, 1, pos0, T, stream_));
+    LS_TRY(ntk_lightning_attention(att_, hv, a_, na, a_ + m.k_off, na, a_ + m.v_off, na, m.log_decay, state, m.heads, m.dim, m.vdim, 1, pos0, T, lscratch_, stream_));
     LS_TRY(ntk_gated_rmsnorm(att_, hv, att_, hv, m.norm, a_ + m.g_off, na, T, hv, eps_, stream_));
     return ntk_dense_linear(mix_, W, att_, hv, m.o.ptr, m.o.dtype, T, W, hv, 0, stream_);
 }
@@ -650,10 +655,22 @@ int LayerStackModel::run_dense_ff(const StackLayer& L, int T) {
 }
 
 // out = h + conv(h), h = layer norm of the stream: the carried inputs in front of the portion's, the convolution, and the portion's last inputs carried on
+// The sublayer output that the stream has not taken yet (owed_) goes in first, in the same launch: the norm after one sublayer and the norm before the next
+// read the same row.  One token: one launch for the whole seam.
 int LayerStackModel::norm_conv(const NormW& nw, const float* canon, float* conv_state, float* out, int T, int pos0) {
     const int W = info_.width;
-    LS_TRY(ntk_layernorm_history(hist_, x_, W, nw.w, nw.b, conv_state, taps_, pos0, T, W, eps_, stream_));
-    return ntk_causal_conv_mix(out, W, hist_, canon, conv_state, taps_, T, W, stream_);
+    const int st = ntk_sandwich_norm_conv(out, W, x_, W, owed_.y, W, owed_.nb.w, owed_.nb.b, nw.w, nw.b, canon, conv_state, hist_, taps_, pos0, T, W, eps_, stream_);
+    owed_.y = nullptr;
+    return st;
+}
+
+// x += norm(owed sublayer output), on its own: after the last layer run, and after every one while the stream is being captured
+int LayerStackModel::settle(int T) {
+    if (!owed_.y) return NTK_OK;
+    const int W = info_.width;
+    const int st = ntk_layernorm(x_, W, owed_.y, W, owed_.nb.w, owed_.nb.b, T, W, eps_, 1, stream_);
+    owed_.y = nullptr;
+    return st;
 }
 
 int LayerStackModel::sequential_layer(const Run& run, const StackLayer& L, int slot, int T, int pos0) {
@@ -662,12 +679,13 @@ int LayerStackModel::sequential_layer(const Run& run, const StackLayer& L, int s
     LS_TRY(norm_conv(L.norm1, L.canon1, conv, h1_, T, pos0));
     if (L.mixer == kMixWindow) LS_TRY(run_window(L, run.cache + (size_t)slot * opt_.max_context * L.att.row(), T, pos0));
     else LS_TRY(run_lightning(L, run.state + (size_t)slot * L.lin.state_floats(), T, pos0));
-    LS_TRY(ntk_layernorm(x_, W, mix_, W, L.norm1b.w, L.norm1b.b, T, W, eps_, 1, stream_));
+    owed_ = Owed{mix_, L.norm1b};
     if (!L.has_mlp) return NTK_OK;
     LS_TRY(norm_conv(L.norm2, L.canon2, conv ? conv + (size_t)(taps_ - 1) * W : nullptr, h2_, T, pos0));
     if (L.mlp_kind == kMlpMoe) LS_TRY(run_moe(L, T, false));
     else LS_TRY(run_dense_ff(L, T));
-    return ntk_layernorm(x_, W, ff_, W, L.norm2b.w, L.norm2b.b, T, W, eps_, 1, stream_);
+    owed_ = Owed{ff_, L.norm2b};
+    return NTK_OK;
 }
 
 int LayerStackModel::parallel_layer(const Run& run, const StackLayer& L, int slot, int T, int pos0) {
@@ -685,8 +703,11 @@ int LayerStackModel::parallel_layer(const Run& run, const StackLayer& L, int slo
 
 int LayerStackModel::portion(int slot, const int* tokens_dev, int T, int pos0, const int* want_dev, int n_want, float* logits_out) {
     const int W = info_.width;
-    LS_TRY(ntk_embed_dense_scaled(x0_, embed_.ptr, embed_.dtype, tokens_dev, T, info_.vocab, W, embed_scale_, stream_));
-    bool x_is_x0 = true;   // until the first layer run writes x_
+    // (the embedding is kept beside the stream only where a repeated span is entered through a projection of both)
+    const bool keep_embedding = has_loop_ && form_.loop_projection;
+    LS_TRY(ntk_embed_dense_scaled(keep_embedding ? x0_ : x_, embed_.ptr, embed_.dtype, tokens_dev, T, info_.vocab, W, embed_scale_, stream_));
+    bool x_is_x0 = keep_embedding;   // until the first layer run writes x_
+    owed_.y = nullptr;
     for (size_t r = 0; r < runs_.size(); ++r) {
         const Run& run = runs_[r];
         const StackLayer& L = layers_[(size_t)run.layer];
@@ -696,8 +717,12 @@ int LayerStackModel::portion(int slot, const int* tokens_dev, int T, int pos0, c
             LS_TRY(ntk_dense_linear(x_, W, cat_, 2 * W, loop_in_.ptr, loop_in_.dtype, T, W, 2 * W, 0, stream_));
             x_is_x0 = false;
         }
-        if (form_.sequential) LS_TRY(sequential_layer(run, L, slot, T, pos0));
-        else LS_TRY(parallel_layer(run, L, slot, T, pos0));
+        if (form_.sequential) {
+            LS_TRY(sequential_layer(run, L, slot, T, pos0));
+            if (r + 1 == runs_.size() || (capture_ && capture_buf_)) LS_TRY(settle(T));
+        } else {
+            LS_TRY(parallel_layer(run, L, slot, T, pos0));
+        }
         if (capture_ && capture_buf_) LS_TRY(ntk_rows_copy(capture_buf_ + r * (size_t)T * W, x_, (long long)T * W, stream_));
     }
     if (n_want > 0) {

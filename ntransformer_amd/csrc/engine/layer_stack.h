@@ -171,9 +171,12 @@ private:
     int run_dense_ff(const StackLayer& L, int T);
     int run_experts(const MoeFeedForward& M, const GatedExperts& ex, const float* h, float* gu, float* act, float* out, int rows, const int* offsets, const int* order, int top);
     int norm_conv(const NormW& nw, const float* canon, float* conv_state, float* out, int T, int pos0);
+    int settle(int T);
     int sequential_layer(const Run& run, const StackLayer& L, int slot, int T, int pos0);
     int parallel_layer(const Run& run, const StackLayer& L, int slot, int T, int pos0);
 
+    struct Owed { const float* y = nullptr; NormW nb; };   // sequential form: a sublayer's output that its norm has yet to add to the stream
+    Owed owed_;
     StackForm form_;
     SeqModelInfo info_;
     std::string err_;
@@ -198,7 +201,7 @@ private:
     // activations
     float *x_ = nullptr, *x0_ = nullptr, *cat_ = nullptr, *h1_ = nullptr, *h2_ = nullptr, *a_ = nullptr, *cq_ = nullptr, *q_ = nullptr, *qf_ = nullptr, *lat_ = nullptr,
           *att_ = nullptr, *kx_ = nullptr, *vx_ = nullptr, *mix_ = nullptr, *wts_ = nullptr, *sg_ = nullptr, *gu_ = nullptr, *act_ = nullptr, *dn_ = nullptr,
-          *sgu_ = nullptr, *sact_ = nullptr, *sdn_ = nullptr, *scratch_ = nullptr, *xw_ = nullptr, *hn_ = nullptr, *hist_ = nullptr, *ff_ = nullptr, *zf_ = nullptr, *wscratch_ = nullptr;
+          *sgu_ = nullptr, *sact_ = nullptr, *sdn_ = nullptr, *scratch_ = nullptr, *xw_ = nullptr, *hn_ = nullptr, *hist_ = nullptr, *ff_ = nullptr, *zf_ = nullptr, *wscratch_ = nullptr, *lscratch_ = nullptr;
     int *ids_ = nullptr, *offsets_ = nullptr, *order_ = nullptr, *where_ = nullptr, *tokens_dev_ = nullptr, *want_dev_ = nullptr;
     int* h_stage_ = nullptr;          // pinned: tokens and wanted places of the pass being launched
     float* logits_ = nullptr;

@@ -72,29 +72,54 @@ __global__ void scale_kernel(float* x, long long n, float s) {
     if (i < n) x[i] *= s;
 }
 
-// mean first, then the mean of the squared deviations (the row is read again: it sits in the cache), then the outputs
-__device__ __forceinline__ void layernorm_row(float* y, const float* xr, const float* w, const float* b, int n, float eps, bool accumulate, float* red) {
+// mean first, then the mean of the squared deviations, then the outputs.  A thread keeps its first LN_KEEP entries (i = tid + 256 k) in registers -- rows up to
+// 4096 wide are read once --; what lies beyond is read again (it sits in the cache).  Returns through (mean, inv); `emit(i, normed value)` writes.
+// Workgroups of NT threads: 256 where a launch has many rows, 1024 where it has few (decoding: a row's entries are then spread over four times the threads,
+// whose loads are in flight together -- a thread's own entries follow each other through load, use and store).
+template <int NT, typename Emit>
+__device__ __forceinline__ void layernorm_row(const float* xr, const float* w, const float* b, int n, float eps, float* red, Emit emit) {
+    constexpr int KEEP = 4096 / NT;
+    float v[KEEP], wv[KEEP], bv[KEEP];
     float s = 0.0f;
-    for (int i = threadIdx.x; i < n; i += 256) s += xr[i];
-    const float mean = block_sum(s, red) / (float)n;
-    float v = 0.0f;
-    for (int i = threadIdx.x; i < n; i += 256) { const float d = xr[i] - mean; v = fmaf(d, d, v); }
-    const float inv = 1.0f / sqrtf(block_sum(v, red) / (float)n + eps);
-    for (int i = threadIdx.x; i < n; i += 256) {
-        float o = (xr[i] - mean) * inv * w[i];
-        if (b) o += b[i];
-        y[i] = accumulate ? y[i] + o : o;
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+        const int i = threadIdx.x + NT * k;
+        v[k] = i < n ? xr[i] : 0.0f;
+        wv[k] = i < n ? w[i] : 0.0f;
+        bv[k] = i < n && b ? b[i] : 0.0f;
+        s += v[k];
     }
+    for (int i = threadIdx.x + NT * KEEP; i < n; i += NT) s += xr[i];
+    const float mean = block_sum(s, red) / (float)n;
+    float q = 0.0f;
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+        const float d = v[k] - mean;
+        if ((int)threadIdx.x + NT * k < n) q = fmaf(d, d, q);
+    }
+    for (int i = threadIdx.x + NT * KEEP; i < n; i += NT) { const float d = xr[i] - mean; q = fmaf(d, d, q); }
+    const float inv = 1.0f / sqrtf(block_sum(q, red) / (float)n + eps);
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+        const int i = threadIdx.x + NT * k;
+        if (i < n) emit(i, (v[k] - mean) * inv * wv[k] + bv[k]);
+    }
+    for (int i = threadIdx.x + NT * KEEP; i < n; i += NT) emit(i, (xr[i] - mean) * inv * w[i] + (b ? b[i] : 0.0f));
 }
 
-__global__ __launch_bounds__(256) void layernorm_kernel(float* y, int ldy, const float* x, int ldx, const float* w, const float* b, int n, float eps, int accumulate) {
+template <int NT>
+__global__ __launch_bounds__(NT) void layernorm_kernel(float* y, int ldy, const float* x, int ldx, const float* w, const float* b, int n, float eps, int accumulate) {
     __shared__ float red[16];
-    layernorm_row(y + (long long)blockIdx.x * ldy, x + (long long)blockIdx.x * ldx, w, b, n, eps, accumulate != 0, red);
+    float* yr = y + (long long)blockIdx.x * ldy;
+    if (accumulate) layernorm_row<NT>(x + (long long)blockIdx.x * ldx, w, b, n, eps, red, [&](int i, float o) { yr[i] += o; });
+    else layernorm_row<NT>(x + (long long)blockIdx.x * ldx, w, b, n, eps, red, [&](int i, float o) { yr[i] = o; });
 }
 
-// rows 0 .. taps-2: the carried inputs (zeros before the sequence's start); rows taps-1 ..: the layer norm of the portion's tokens
-__global__ __launch_bounds__(256) void layernorm_history_kernel(float* hist, const float* x, int ldx, const float* w, const float* b, const float* state, int taps,
-                                                                int pos0, int n, float eps) {
+// rows 0 .. taps-2: the carried inputs (zeros before the sequence's start); rows taps-1 ..: the layer norm of the portion's tokens.  With add_y the stream row
+// first takes the sublayer output that is still owed to it, x[t] += layer norm of add_y[t] (weights add_w / add_b): the norm after one sublayer and the norm
+// before the next in one pass over the row (a thread reads back only what it wrote itself).
+__global__ __launch_bounds__(256) void layernorm_history_kernel(float* hist, float* x, int ldx, const float* w, const float* b, const float* state, int taps,
+                                                                int pos0, int n, float eps, const float* add_y, int ldy, const float* add_w, const float* add_b) {
     __shared__ float red[16];
     const int r = blockIdx.x;
     float* o = hist + (long long)r * n;
@@ -103,7 +128,30 @@ __global__ __launch_bounds__(256) void layernorm_history_kernel(float* hist, con
         for (int i = threadIdx.x; i < n; i += 256) o[i] = before ? 0.0f : state[(long long)r * n + i];
         return;
     }
-    layernorm_row(o, x + (long long)(r - (taps - 1)) * ldx, w, b, n, eps, false, red);
+    float* xr = x + (long long)(r - (taps - 1)) * ldx;
+    if (add_y) layernorm_row<256>(add_y + (long long)(r - (taps - 1)) * ldy, add_w, add_b, n, eps, red, [&](int i, float v) { xr[i] += v; });
+    layernorm_row<256>(xr, w, b, n, eps, red, [&](int i, float v) { o[i] = v; });
+}
+
+// one token (decoding), one workgroup: the owed sublayer output onto the stream, the norm, the convolution over the carried inputs and their shift -- every
+// channel's history belongs to the thread that owns the channel.  Same sums in the same order as the two launches of a longer portion.
+constexpr int kStepThreads = 1024;
+__global__ __launch_bounds__(kStepThreads) void sandwich_step_kernel(float* out, float* x, const float* w, const float* b, const float* canon, float* state, int taps, int pos0,
+                                                            int n, float eps, const float* add_y, const float* add_w, const float* add_b) {
+    __shared__ float red[16];
+    if (add_y) layernorm_row<kStepThreads>(add_y, add_w, add_b, n, eps, red, [&](int i, float v) { x[i] += v; });
+    layernorm_row<kStepThreads>(x, w, b, n, eps, red, [&](int i, float h) {
+        const float* cw = canon + (long long)i * taps;
+        float s = 0.0f;
+        for (int j = 0; j < taps - 1; ++j) {
+            const float hj = pos0 - (taps - 1) + j >= 0 ? state[(long long)j * n + i] : 0.0f;
+            s = fmaf(cw[j], hj, s);
+            if (j > 0) state[(long long)(j - 1) * n + i] = hj;
+        }
+        s = fmaf(cw[taps - 1], h, s);
+        if (taps > 1) state[(long long)(taps - 2) * n + i] = h;
+        out[i] = h + s;
+    });
 }
 
 // blocks y < T: out[y] = hist[taps-1+y] + sum_j w[:, j] * hist[y+j] (j ascending); blocks y >= T: the carried rows for the next portion
@@ -116,36 +164,38 @@ __global__ void causal_conv_mix_kernel(float* out, int ldo, const float* hist, c
     out[(long long)y * ldo + c] = hist[(long long)(y + taps - 1) * n + c] + s;
 }
 
-__global__ __launch_bounds__(256) void polynorm_kernel(float* y, int ldy, const float* z, int ldz, const float* coef, int n, float eps) {
+__global__ __launch_bounds__(1024) void polynorm_kernel(float* y, int ldy, const float* z, int ldz, const float* coef, int n, float eps) {
     __shared__ float red[16];
     const float* zr = z + (long long)blockIdx.x * ldz;
     float s2 = 0.0f, s4 = 0.0f, s6 = 0.0f;
-    for (int i = threadIdx.x; i < n; i += 256) {
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
         const float v = zr[i], v2 = v * v, v3 = v2 * v;
         s2 += v2; s4 = fmaf(v2, v2, s4); s6 = fmaf(v3, v3, s6);
     }
     s2 = block_sum(s2, red); s4 = block_sum(s4, red); s6 = block_sum(s6, red);
     const float i1 = coef[0] / sqrtf(s2 / (float)n + eps), i2 = coef[1] / sqrtf(s4 / (float)n + eps), i3 = coef[2] / sqrtf(s6 / (float)n + eps), e = coef[3];
     float* o = y + (long long)blockIdx.x * ldy;
-    for (int i = threadIdx.x; i < n; i += 256) {
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
         const float v = zr[i], v2 = v * v, v3 = v2 * v;
         o[i] = i1 * v + i2 * v2 + i3 * v3 + e;
     }
 }
 
-__global__ __launch_bounds__(256) void gated_rmsnorm_kernel(float* y, int ldy, const float* x, int ldx, const float* w, const float* g, int ldg, int n, float eps) {
+__global__ __launch_bounds__(1024) void gated_rmsnorm_kernel(float* y, int ldy, const float* x, int ldx, const float* w, const float* g, int ldg, int n, float eps) {
     __shared__ float red[16];
     const float* xr = x + (long long)blockIdx.x * ldx;
     float ss = 0.0f;
-    for (int i = threadIdx.x; i < n; i += 256) ss = fmaf(xr[i], xr[i], ss);
+    for (int i = threadIdx.x; i < n; i += blockDim.x) ss = fmaf(xr[i], xr[i], ss);
     const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)n + eps);
     float* o = y + (long long)blockIdx.x * ldy;
-    for (int i = threadIdx.x; i < n; i += 256) {
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
         float v = xr[i] * inv * w[i];
         if (g) v *= 1.0f / (1.0f + expf(-g[(long long)blockIdx.x * ldg + i]));
         o[i] = v;
     }
 }
+
+constexpr int kFewRows = 32;   // up to this many rows a row kernel runs workgroups of 1024 threads
 
 }  // namespace ntk
 
@@ -218,7 +268,8 @@ int ntk_layernorm(float* y, int ldy, const float* x, int ldx, const float* w, co
     if (!y || !x || !w) return NTK_E_NULL;
     if (T < 0 || n <= 0 || ldy < n || ldx < n) return NTK_E_SHAPE;
     if (T == 0) return NTK_OK;
-    hipLaunchKernelGGL(layernorm_kernel, dim3(T), dim3(256), 0, resolve_stream(stream), y, ldy, x, ldx, w, b, n, eps, accumulate);
+    if (T <= kFewRows) hipLaunchKernelGGL(layernorm_kernel<1024>, dim3(T), dim3(1024), 0, resolve_stream(stream), y, ldy, x, ldx, w, b, n, eps, accumulate);
+    else hipLaunchKernelGGL(layernorm_kernel<256>, dim3(T), dim3(256), 0, resolve_stream(stream), y, ldy, x, ldx, w, b, n, eps, accumulate);
     return last_launch_status();
 }
 
@@ -227,8 +278,26 @@ int ntk_layernorm_history(float* hist, const float* x, int ldx, const float* w, 
     if (!hist || !x || !w || (taps > 1 && !state)) return NTK_E_NULL;
     if (T < 0 || n <= 0 || ldx < n || taps < 1 || pos0 < 0) return NTK_E_SHAPE;
     if (T == 0) return NTK_OK;
-    hipLaunchKernelGGL(layernorm_history_kernel, dim3(T + taps - 1), dim3(256), 0, resolve_stream(stream), hist, x, ldx, w, b, state, taps, pos0, n, eps);
+    hipLaunchKernelGGL(layernorm_history_kernel, dim3(T + taps - 1), dim3(256), 0, resolve_stream(stream), hist, const_cast<float*>(x), ldx, w, b, state, taps, pos0, n,
+                       eps, (const float*)nullptr, 0, (const float*)nullptr, (const float*)nullptr);
     return last_launch_status();
+}
+
+int ntk_sandwich_norm_conv(float* out, int ldo, float* x, int ldx, const float* add_y, int ldy, const float* add_w, const float* add_b, const float* w, const float* b,
+                           const float* canon, float* state, float* hist, int taps, int pos0, int T, int n, float eps, void* stream) {
+    if (!out || !x || !w || !canon || (taps > 1 && !state) || (add_y && !add_w)) return NTK_E_NULL;
+    if (T < 0 || n <= 0 || ldx < n || ldo < n || (add_y && ldy < n) || taps < 1 || pos0 < 0) return NTK_E_SHAPE;
+    if (T == 0) return NTK_OK;
+    hipStream_t s = resolve_stream(stream);
+    if (T == 1) {
+        hipLaunchKernelGGL(sandwich_step_kernel, dim3(1), dim3(kStepThreads), 0, s, out, x, w, b, canon, state, taps, pos0, n, eps, add_y, add_w, add_b);
+        return last_launch_status();
+    }
+    if (!hist) return NTK_E_NULL;
+    hipLaunchKernelGGL(layernorm_history_kernel, dim3(T + taps - 1), dim3(256), 0, s, hist, x, ldx, w, b, (const float*)state, taps, pos0, n, eps, add_y, ldy, add_w, add_b);
+    const int st = last_launch_status();
+    if (st != NTK_OK) return st;
+    return ntk_causal_conv_mix(out, ldo, hist, canon, state, taps, T, n, stream);
 }
 
 int ntk_causal_conv_mix(float* out, int ldo, const float* hist, const float* w, float* state, int taps, int T, int n, void* stream) {
@@ -243,7 +312,7 @@ int ntk_polynorm(float* y, int ldy, const float* z, int ldz, const float* coef, 
     if (!y || !z || !coef) return NTK_E_NULL;
     if (T < 0 || n <= 0 || ldy < n || ldz < n) return NTK_E_SHAPE;
     if (T == 0) return NTK_OK;
-    hipLaunchKernelGGL(polynorm_kernel, dim3(T), dim3(256), 0, resolve_stream(stream), y, ldy, z, ldz, coef, n, eps);
+    hipLaunchKernelGGL(polynorm_kernel, dim3(T), dim3(T <= kFewRows ? 1024 : 256), 0, resolve_stream(stream), y, ldy, z, ldz, coef, n, eps);
     return last_launch_status();
 }
 
@@ -251,6 +320,6 @@ int ntk_gated_rmsnorm(float* y, int ldy, const float* x, int ldx, const float* w
     if (!y || !x || !w) return NTK_E_NULL;
     if (T < 0 || n <= 0 || ldy < n || ldx < n || (g && ldg < n)) return NTK_E_SHAPE;
     if (T == 0) return NTK_OK;
-    hipLaunchKernelGGL(gated_rmsnorm_kernel, dim3(T), dim3(256), 0, resolve_stream(stream), y, ldy, x, ldx, w, g, ldg, n, eps);
+    hipLaunchKernelGGL(gated_rmsnorm_kernel, dim3(T), dim3(T <= kFewRows ? 1024 : 256), 0, resolve_stream(stream), y, ldy, x, ldx, w, g, ldg, n, eps);
     return last_launch_status();
 }

@@ -5,9 +5,15 @@
 //     S_new = exp(n L) S + sum_j exp((n - 1 - j) L) k_j v_j^T                  (n = tokens of the chunk)
 // -- only non-negative powers of the decay occur, so nothing overflows however small it is.  A workgroup owns one head and a slab of 64 value columns and
 // keeps its [dn][64] slice of the state in LDS across the chunks; the state is read from memory at the start (zeros when the sequence starts here) and written
-// back at the end.  One token (decoding) is a chunk of one: the state slice is read, updated and written once.
-// Thread tiles are 4 x 4 (scores: tokens x tokens; outputs: tokens x columns) and (dn / 16) x 4 (state rows x columns); q, k and v pass through silu on
-// their way into LDS when the caller asks for it.
+// back at the end.  Thread tiles are 4 x 4 (scores: tokens x tokens; outputs: tokens x columns) and (dn / 16) x 4 (state rows x columns); q, k and v pass
+// through silu on their way into LDS when the caller asks for it.
+// Three forms of the same sums:
+//   * few tokens (decoding, up to kStepRows): lightning_step_kernel keeps its state slice in REGISTERS (thread = (rows d = part + 4 r, one value column)), walks the
+//     tokens one by one -- S = decay S + k v^T, o = S^T q with the four row parts added through LDS -- and writes the slice back: state bytes once in, once out;
+//   * one chunk or no scratch: lightning_chunk_kernel<C, kWhole>, the walk described above by one workgroup per (head, value slab);
+//   * long portions with scratch: the chunks run side by side.  kLocal: every (chunk, head, slab) forms its own sum_j exp((n - 1 - j) L) k_j v_j^T;
+//     lightning_scan_kernel then walks the chunks per state element (S_c = exp(n L) S_(c-1) + local_c, leaving S_(c-1) where local_c was) and writes the final
+//     state; kOutputs: every (chunk, head, slab) forms its outputs from its chunk's scores and the state before it.
 #include "common.hip.h"
 #include "../../include/ntk_layers.h"
 
@@ -23,13 +29,16 @@ struct LightArgs {
     const float* log_decay;
     float* state;
     int H, dn, dv, silu, pos0, T;
+    float* scratch;
 };
 
 __device__ __forceinline__ float decay_pow(float L, int n) { return n == 0 ? 1.0f : expf((float)n * L); }
 __device__ __forceinline__ float maybe_silu(float x, int on) { return on ? x / (1.0f + expf(-x)) : x; }
 
-template <int C>
-__global__ __launch_bounds__(256) void lightning_attention_kernel(const LightArgs a) {
+enum ChunkMode { kWhole = 0, kLocal = 1, kOutputs = 2 };
+
+template <int C, int MODE>
+__global__ __launch_bounds__(256) void lightning_chunk_kernel(const LightArgs a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int DP = (a.dn + 15) & ~15;              // state rows, padded (the padding stays zero)
     const int LQ = DP + 1;                         // row length of the q / k chunks
@@ -42,14 +51,17 @@ __global__ __launch_bounds__(256) void lightning_attention_kernel(const LightArg
     const int h = blockIdx.x, v0 = blockIdx.y * LV, nv = min(LV, a.dv - v0);
     const int tid = threadIdx.x;
     const float L = a.log_decay[h];
-    float* sg = a.state + ((long long)h * a.dn) * a.dv + v0;
+    // kWhole: the sequence's state; kLocal / kOutputs: this chunk's slot of the scratch [chunks][H][dn][dv] (written / read)
+    float* sg = (MODE == kWhole ? a.state : a.scratch + (long long)blockIdx.z * a.H * a.dn * a.dv) + ((long long)h * a.dn) * a.dv + v0;
     for (int e = tid; e < DP * LV; e += 256) {
         const int d = e / LV, c = e % LV;
-        Ss[e] = (a.pos0 > 0 && d < a.dn && c < nv) ? sg[(long long)d * a.dv + c] : 0.0f;
+        const bool have = MODE == kOutputs || (MODE == kWhole && a.pos0 > 0);
+        Ss[e] = (have && d < a.dn && c < nv) ? sg[(long long)d * a.dv + c] : 0.0f;
     }
     const int ti = tid / 16, tj = tid % 16;        // 16 x 16 thread grid
     constexpr int RI = C / 16;                     // token rows per thread (C = 64: 4, C = 32: 2)
-    for (int t0 = 0; t0 < a.T; t0 += C) {
+    const int t_first = MODE == kWhole ? 0 : (int)blockIdx.z * C, t_last = MODE == kWhole ? a.T : min(a.T, t_first + C);
+    for (int t0 = t_first; t0 < t_last; t0 += C) {
         const int n = min(C, a.T - t0);
         const int nr = min(C, (n + RI - 1) / RI * RI);   // rows a thread tile may touch: the chunk's tokens rounded up to whole tiles
         __syncthreads();                           // the last chunk's readers are done (and the state slice is in place)
@@ -70,7 +82,7 @@ __global__ __launch_bounds__(256) void lightning_attention_kernel(const LightArg
         }
         __syncthreads();
         // ---- decayed scores inside the chunk: thread (ti, tj) owns tokens i = ti * RI + r against j = tj * RI + c
-        if (ti * RI < n && tj <= ti) {
+        if (MODE != kLocal && ti * RI < n && tj <= ti) {
             float s[RI][RI];
 #pragma unroll
             for (int r = 0; r < RI; ++r)
@@ -92,15 +104,10 @@ __global__ __launch_bounds__(256) void lightning_attention_kernel(const LightArg
                     const int i = ti * RI + r, j = tj * RI + c;
                     Ps[i * (C + 1) + j] = j <= i ? s[r][c] * decay_pow(L, i - j) : 0.0f;
                 }
-        } else if (ti * RI < n) {
-#pragma unroll
-            for (int r = 0; r < RI; ++r)
-#pragma unroll
-                for (int c = 0; c < RI; ++c) Ps[(ti * RI + r) * (C + 1) + tj * RI + c] = 0.0f;
         }
         __syncthreads();
-        // ---- outputs: thread (ti, tj) owns tokens ti * RI + r and columns tj * 4 + c
-        if (ti * RI < n) {
+        // ---- outputs: thread (ti, tj) owns tokens ti * RI + r and columns tj * 4 + c (the scores above the diagonal tiles are never read)
+        if (MODE != kLocal && ti * RI < n) {
             float o[RI][4], u[RI][4];
 #pragma unroll
             for (int r = 0; r < RI; ++r)
@@ -134,6 +141,7 @@ __global__ __launch_bounds__(256) void lightning_attention_kernel(const LightArg
                     if (tj * 4 + c < nv) op[c] = fmaf(w, u[r][c], o[r][c]);
             }
         }
+        if (MODE == kOutputs) break;
         __syncthreads();                           // every reader of the old state slice is done
         // ---- the state: thread (ti, tj) owns rows d = ti + 16 r and columns tj * 4 + c; every token's value row is read once for all of them
         {
@@ -162,6 +170,7 @@ __global__ __launch_bounds__(256) void lightning_attention_kernel(const LightArg
                 }
         }
     }
+    if (MODE == kOutputs) return;
     __syncthreads();
     for (int e = tid; e < DP * LV; e += 256) {
         const int d = e / LV, c = e % LV;
@@ -169,29 +178,126 @@ __global__ __launch_bounds__(256) void lightning_attention_kernel(const LightArg
     }
 }
 
+// one thread per state element: the chunks' local sums become the states BEFORE their chunks, the sequence's state moves on by the whole portion
+template <int C>
+__global__ __launch_bounds__(256) void lightning_scan_kernel(const LightArgs a) {
+    const long long per = (long long)a.H * a.dn * a.dv;
+    const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (e >= per) return;
+    const float L = a.log_decay[e / ((long long)a.dn * a.dv)];
+    float S = a.pos0 > 0 ? a.state[e] : 0.0f;
+    const int chunks = (a.T + C - 1) / C;
+    const float wfull = decay_pow(L, C);
+    for (int c = 0; c < chunks; ++c) {
+        const float local = a.scratch[c * per + e];
+        a.scratch[c * per + e] = S;
+        const int n = min(C, a.T - c * C);
+        S = fmaf(n == C ? wfull : decay_pow(L, n), S, local);
+    }
+    a.state[e] = S;
+}
+
+// few tokens: the state slice of (head, 64 value columns) in registers, rows d = part + 4 r of wave `part`; tokens one by one
+constexpr int kStepRows = 8;
+template <int NR>
+__global__ __launch_bounds__(256) void lightning_step_kernel(const LightArgs a) {
+    __shared__ float qs[256], ks[256], red[4][LV];
+    const int h = blockIdx.x, v0 = blockIdx.y * LV, col = threadIdx.x & 63, part = threadIdx.x >> 6;
+    const bool live = v0 + col < a.dv;
+    const float lam = decay_pow(a.log_decay[h], 1);
+    float* sg = a.state + ((long long)h * a.dn) * a.dv + v0 + col;
+    float S[NR];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        const int d = part + 4 * r;
+        S[r] = (a.pos0 > 0 && live && d < a.dn) ? sg[(long long)d * a.dv] : 0.0f;
+    }
+    for (int t = 0; t < a.T; ++t) {
+        __syncthreads();                           // the last token's readers are done
+        if ((int)threadIdx.x < a.dn) {
+            qs[threadIdx.x] = maybe_silu(a.q[(long long)t * a.ldq + h * a.dn + threadIdx.x], a.silu);
+            ks[threadIdx.x] = maybe_silu(a.k[(long long)t * a.ldk + h * a.dn + threadIdx.x], a.silu);
+        }
+        const float vv = live ? maybe_silu(a.v[(long long)t * a.ldv + h * a.dv + v0 + col], a.silu) : 0.0f;
+        __syncthreads();
+        float o = 0.0f;
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int d = part + 4 * r;
+            if (d < a.dn) {
+                S[r] = fmaf(lam, S[r], ks[d] * vv);
+                o = fmaf(S[r], qs[d], o);
+            }
+        }
+        red[part][col] = o;
+        __syncthreads();
+        if (part == 0 && live) a.out[(long long)t * a.ldo + h * a.dv + v0 + col] = (red[0][col] + red[1][col]) + (red[2][col] + red[3][col]);
+    }
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        const int d = part + 4 * r;
+        if (live && d < a.dn) sg[(long long)d * a.dv] = S[r];
+    }
+}
+
 }  // namespace ntk
 
 using namespace ntk;
 
+static int light_chunk(int dn) { return dn > 128 ? 32 : 64; }   // chunk length: the LDS of two [C][dn] chunks, the value slab, the state slice and the scores
+
+size_t ntk_lightning_attention_scratch(int T, int H, int dn, int dv) {
+    if (T <= 0 || H <= 0 || dn <= 0 || dv <= 0) return 0;
+    const int C = light_chunk(dn);
+    return T > C ? (size_t)((T + C - 1) / C) * H * dn * dv : 0;
+}
+
 int ntk_lightning_attention(float* out, int ldo, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* log_decay, float* state,
-                            int H, int dn, int dv, int silu, int pos0, int T, void* stream) {
+                            int H, int dn, int dv, int silu, int pos0, int T, float* scratch, void* stream) {
     if (!out || !q || !k || !v || !log_decay || !state) return NTK_E_NULL;
     if (T < 0 || H <= 0 || dn <= 0 || dn > 256 || dv <= 0 || pos0 < 0) return NTK_E_SHAPE;
     if (ldo < H * dv || ldq < H * dn || ldk < H * dn || ldv < H * dv) return NTK_E_SHAPE;
     if (T == 0) return NTK_OK;
-    LightArgs a{out, ldo, q, ldq, k, ldk, v, ldv, log_decay, state, H, dn, dv, silu, pos0, T};
+    LightArgs a{out, ldo, q, ldq, k, ldk, v, ldv, log_decay, state, H, dn, dv, silu, pos0, T, scratch};
+    hipStream_t s = resolve_stream(stream);
+    const int slabs = (dv + LV - 1) / LV;
+    if (T <= kStepRows) {
+        const dim3 grid(H, slabs);
+        if (dn <= 64) hipLaunchKernelGGL(lightning_step_kernel<16>, grid, dim3(256), 0, s, a);
+        else if (dn <= 128) hipLaunchKernelGGL(lightning_step_kernel<32>, grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL(lightning_step_kernel<64>, grid, dim3(256), 0, s, a);
+        return last_launch_status();
+    }
     const int DP = (dn + 15) & ~15;
-    const int C = dn > 128 ? 32 : 64;          // chunk length: the LDS of two [C][dn] chunks, the value slab, the state slice and the scores
+    const int C = light_chunk(dn);
     const size_t lds = ((size_t)2 * C * (DP + 1) + (size_t)C * LV + (size_t)DP * LV + (size_t)C * (C + 1) + C) * sizeof(float);
     if (lds > 156 * 1024) return NTK_E_SHAPE;
     static bool raised = false;   // (idempotent: a race sets the same attribute twice)
     if (!raised) {
-        NTK_HIP_TRY(hipFuncSetAttribute((const void*)lightning_attention_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
-        NTK_HIP_TRY(hipFuncSetAttribute((const void*)lightning_attention_kernel<32>, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
+        NTK_HIP_TRY(hipFuncSetAttribute((const void*)lightning_chunk_kernel<64, kWhole>, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
+        NTK_HIP_TRY(hipFuncSetAttribute((const void*)lightning_chunk_kernel<64, kLocal>, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
+        NTK_HIP_TRY(hipFuncSetAttribute((const void*)lightning_chunk_kernel<64, kOutputs>, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
+        NTK_HIP_TRY(hipFuncSetAttribute((const void*)lightning_chunk_kernel<32, kWhole>, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
+        NTK_HIP_TRY(hipFuncSetAttribute((const void*)lightning_chunk_kernel<32, kLocal>, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
+        NTK_HIP_TRY(hipFuncSetAttribute((const void*)lightning_chunk_kernel<32, kOutputs>, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
         raised = true;
     }
-    const dim3 grid(H, (dv + LV - 1) / LV);
-    if (C == 64) hipLaunchKernelGGL(lightning_attention_kernel<64>, grid, dim3(256), lds, resolve_stream(stream), a);
-    else hipLaunchKernelGGL(lightning_attention_kernel<32>, grid, dim3(256), lds, resolve_stream(stream), a);
+    if (!scratch || T <= C) {
+        const dim3 grid(H, slabs);
+        if (C == 64) hipLaunchKernelGGL((lightning_chunk_kernel<64, kWhole>), grid, dim3(256), lds, s, a);
+        else hipLaunchKernelGGL((lightning_chunk_kernel<32, kWhole>), grid, dim3(256), lds, s, a);
+        return last_launch_status();
+    }
+    const dim3 grid(H, slabs, (T + C - 1) / C);
+    const unsigned scan_blocks = (unsigned)(((long long)H * dn * dv + 255) / 256);
+    if (C == 64) {
+        hipLaunchKernelGGL((lightning_chunk_kernel<64, kLocal>), grid, dim3(256), lds, s, a);
+        hipLaunchKernelGGL(lightning_scan_kernel<64>, dim3(scan_blocks), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((lightning_chunk_kernel<64, kOutputs>), grid, dim3(256), lds, s, a);
+    } else {
+        hipLaunchKernelGGL((lightning_chunk_kernel<32, kLocal>), grid, dim3(256), lds, s, a);
+        hipLaunchKernelGGL(lightning_scan_kernel<32>, dim3(scan_blocks), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((lightning_chunk_kernel<32, kOutputs>), grid, dim3(256), lds, s, a);
+    }
     return last_launch_status();
 }

@@ -231,7 +231,8 @@ __global__ __launch_bounds__(256) void window_attention_kernel(const WinArgs a) 
     }
 }
 
-// merge of the partial states of one (token, head) row, one wave per row: the states' weights first, then lane = column sums over the states in order
+// merge of the partial states of one (token, head) row, one wave per row: lane = part for the weights exp(max_s - max) and the sum (splits <= 64), then
+// lane = column for the weighted vectors, the parts in order with their loads independent of each other
 template <int M>
 __global__ __launch_bounds__(64) void window_attention_merge_kernel(const WinArgs a) {
     const int lane = threadIdx.x, row = blockIdx.x;       // row = t * H + h
@@ -240,19 +241,27 @@ __global__ __launch_bounds__(64) void window_attention_merge_kernel(const WinArg
     for (int m = 0; m < M; ++m) {
         const float* st = a.scratch + ((long long)row * a.splits * M + m) * (2 + a.dv);
         const long long step = (long long)M * (2 + a.dv);
-        float mm = -INFINITY;
-        for (int s = 0; s < a.splits; ++s) mm = fmaxf(mm, st[s * step]);
-        float L = 0.0f;
+        const float ms = lane < a.splits ? st[lane * step] : -INFINITY;
+        const float ls = lane < a.splits ? st[lane * step + 1] : 0.0f;
+        const float mm = wave_max(ms);
+        const float w = ms == -INFINITY ? 0.0f : expf(ms - mm);
+        const float L = wave_sum(w * ls);
 #pragma unroll
         for (int c = 0; c < WMAXC; ++c) r[m][c] = 0.0f;
-        for (int s = 0; s < a.splits; ++s) {
-            const float ms = st[s * step];
-            if (ms == -INFINITY) continue;
-            const float w = expf(ms - mm);
-            L = fmaf(w, st[s * step + 1], L);
+        const int nc = (a.dv + WSLAB - 1) / WSLAB;
+        for (int s0 = 0; s0 < a.splits; s0 += 8) {       // eight parts' loads in flight before the first is used
+            for (int c = 0; c < nc; ++c) {
+                float x[8];
 #pragma unroll
-            for (int c = 0; c < WMAXC; ++c)
-                if (c * WSLAB + lane < a.dv) r[m][c] = fmaf(w, st[s * step + 2 + c * WSLAB + lane], r[m][c]);
+                for (int u = 0; u < 8; ++u) x[u] = (s0 + u < a.splits && c * WSLAB + lane < a.dv) ? st[(s0 + u) * step + 2 + c * WSLAB + lane] : 0.0f;
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const float ws = __shfl(w, (s0 + u) & 63, 64);
+#pragma unroll
+                    for (int cc = 0; cc < WMAXC; ++cc)
+                        if (cc == c) r[m][cc] = fmaf(ws, x[u], r[m][cc]);
+                }
+            }
         }
         const float inv = L > 0.0f ? 1.0f / L : 0.0f;
 #pragma unroll

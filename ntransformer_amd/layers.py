@@ -64,13 +64,16 @@ def _bind():
     L.ntk_layernorm.argtypes = [vp, i, vp, i, vp, vp, i, i, f, i, vp]
     L.ntk_layernorm_history.argtypes = [vp, vp, i, vp, vp, vp, i, i, i, i, f, vp]
     L.ntk_causal_conv_mix.argtypes = [vp, i, vp, vp, vp, i, i, i, vp]
+    L.ntk_sandwich_norm_conv.argtypes = [vp, i, vp, i, vp, i, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, vp]
     L.ntk_polynorm.argtypes = [vp, i, vp, i, vp, i, i, f, vp]
     L.ntk_gated_rmsnorm.argtypes = [vp, i, vp, i, vp, vp, i, i, i, f, vp]
     L.ntk_window_prepare.argtypes = [vp, i, vp, i, vp, i, vp, i, i, i, i, i, i, C.POINTER(Rotary), i, i, vp]
     L.ntk_window_attention_scratch.argtypes = [i, i, i, i, i]
     L.ntk_window_attention_scratch.restype = C.c_size_t
     L.ntk_window_attention.argtypes = [C.POINTER(WindowAttentionDesc), vp]
-    L.ntk_lightning_attention.argtypes = [vp, i, vp, i, vp, i, vp, i, vp, vp, i, i, i, i, i, i, vp]
+    L.ntk_lightning_attention.argtypes = [vp, i, vp, i, vp, i, vp, i, vp, vp, i, i, i, i, i, i, vp, vp]
+    L.ntk_lightning_attention_scratch.argtypes = [i, i, i, i]
+    L.ntk_lightning_attention_scratch.restype = C.c_size_t
     L.ntk_moe_route_ex.argtypes = [vp, vp, vp, vp, i, vp, vp, i, i, i, i, C.POINTER(RouteDesc), vp]
     L.ntk_glu.argtypes = [vp, vp, i, i, f, f, f, vp]
     L.ntk_moe_sum.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, vp]
@@ -267,6 +270,22 @@ def norm_conv(x: np.ndarray, w: np.ndarray, b: np.ndarray, eps: float, canon: np
     return out.numpy(np.float32, T * n).reshape(T, n), sb.numpy(np.float32, max(taps - 1, 1) * n).reshape(-1, n)[:taps - 1]
 
 
+def sandwich_norm_conv(x: np.ndarray, w: np.ndarray, b: np.ndarray, eps: float, canon: np.ndarray, state: Optional[np.ndarray], pos0: int,
+                       owed: Optional[np.ndarray] = None, owed_w: Optional[np.ndarray] = None, owed_b: Optional[np.ndarray] = None):
+    """the seam between two sublayers in one call: x += layer norm of `owed`; h = layer norm of x; -> (h + conv(h), x, the new carried inputs)"""
+    L = _bind()
+    T, n = x.shape
+    taps = canon.shape[1]
+    xb, wb, bb, cb = _f(x), _f(w), _f(b), _f(canon)
+    sb = _f(state) if state is not None else DeviceBuffer.zeros(max(taps - 1, 1) * n * 4)
+    ob, owb, obb = (_f(owed), _f(owed_w), _f(owed_b)) if owed is not None else (None, None, None)
+    hist, out = DeviceBuffer.zeros((T + taps - 1) * n * 4), DeviceBuffer.zeros(T * n * 4)
+    check(L.ntk_sandwich_norm_conv(out.ptr, n, xb.ptr, n, ob.ptr if ob else None, n, owb.ptr if ob else None, obb.ptr if ob else None, wb.ptr, bb.ptr, cb.ptr, sb.ptr,
+                                   hist.ptr, taps, pos0, T, n, eps, None), "ntk_sandwich_norm_conv")
+    return (out.numpy(np.float32, T * n).reshape(T, n), xb.numpy(np.float32, T * n).reshape(T, n),
+            sb.numpy(np.float32, max(taps - 1, 1) * n).reshape(-1, n)[:taps - 1])
+
+
 def polynorm(z: np.ndarray, coef, eps: float) -> np.ndarray:
     L = _bind()
     T, n = z.shape
@@ -314,8 +333,10 @@ def window_attention(q: np.ndarray, cache: np.ndarray, H: int, G: int, maps: int
     return out.numpy(np.float32, T * H * dv).reshape(T, H * dv)
 
 
-def lightning_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, decay, H: int, dn: int, dv: int, pos0: int, state: Optional[np.ndarray] = None, silu: bool = True):
-    """-> (out [T, H * dv], state [H, dn, dv]); state: what an earlier portion left (ignored when pos0 == 0)"""
+def lightning_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, decay, H: int, dn: int, dv: int, pos0: int, state: Optional[np.ndarray] = None, silu: bool = True,
+                        side_by_side: bool = True):
+    """-> (out [T, H * dv], state [H, dn, dv]); state: what an earlier portion left (ignored when pos0 == 0); side_by_side: give the scratch that lets the
+    chunks of a long portion run in parallel"""
     L = _bind()
     T = q.shape[0]
     qb, kb, vb = _f(q), _f(k), _f(v)
@@ -323,8 +344,10 @@ def lightning_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, decay, H: i
         lb = _f(np.log(np.asarray(decay, np.float64)))
     sb = _f(state) if state is not None else DeviceBuffer.from_numpy(np.full(H * dn * dv, np.nan, np.float32))
     out = DeviceBuffer.zeros(T * H * dv * 4)
-    check(L.ntk_lightning_attention(out.ptr, H * dv, qb.ptr, q.shape[1], kb.ptr, k.shape[1], vb.ptr, v.shape[1], lb.ptr, sb.ptr, H, dn, dv, int(silu), pos0, T, None),
-          "ntk_lightning_attention")
+    ns = int(L.ntk_lightning_attention_scratch(T, H, dn, dv)) if side_by_side else 0
+    scr = DeviceBuffer.from_numpy(np.full(ns, np.nan, np.float32)) if ns else None
+    check(L.ntk_lightning_attention(out.ptr, H * dv, qb.ptr, q.shape[1], kb.ptr, k.shape[1], vb.ptr, v.shape[1], lb.ptr, sb.ptr, H, dn, dv, int(silu), pos0, T,
+                                    scr.ptr if scr else None, None), "ntk_lightning_attention")
     return out.numpy(np.float32, T * H * dv).reshape(T, H * dv), sb.numpy(np.float32, H * dn * dv).reshape(H, dn, dv)
 
 

@@ -105,6 +105,38 @@ def test_added_convolution_carries_its_last_inputs_across_portions(taps):
     assert rel(o, 1.25 * O.layer_norm(t64(x), t64(w), t64(b), 1e-5)) < 1e-6
 
 
+@pytest.mark.parametrize("taps", [1, 2, 4])
+@pytest.mark.parametrize("n", [70, 1000, 4500])
+def test_the_seam_between_sublayers_in_one_call(taps, n):
+    """the owed sublayer output onto the stream, the next norm, the convolution and its carried inputs: token by token (one launch each), in portions
+    (two launches), and against the pieces one after the other; rows wider than a thread keeps in registers"""
+    from ntransformer_amd import layers as Lr
+    g = np.random.default_rng(taps + n)
+    T = 9
+    x = (g.standard_normal((T, n)) * 2).astype(np.float32)
+    y = (g.standard_normal((T, n)) * 3 + 1).astype(np.float32)
+    w, b, ow, ob = ((k + 0.2 * g.standard_normal(n)).astype(np.float32) for k in (1, 0, 1, 0))
+    cw = O.bf16_round(torch.tensor(0.5 * g.standard_normal((n, taps)))).numpy().astype(np.float32)
+    xs = t64(x) + O.layer_norm(t64(y), t64(ow), t64(ob), 1e-5)
+    ref, last = O.conv_added(O.layer_norm(xs, t64(w), t64(b), 1e-5), t64(cw))
+    garbage = np.full((max(taps - 1, 1), n), 1e6, np.float32)
+    for cuts in ([T], [1] * T, [1, 3, 1, 4]):
+        outs, news, at, st = [], [], 0, garbage.copy()
+        for k in cuts:
+            o, xn, st2 = Lr.sandwich_norm_conv(x[at:at + k], w, b, 1e-5, cw, st, at, owed=y[at:at + k], owed_w=ow, owed_b=ob)
+            if taps > 1:
+                st = st2
+            outs.append(o)
+            news.append(xn)
+            at += k
+        assert rel(np.concatenate(outs), ref) < 1e-6, cuts
+        assert rel(np.concatenate(news), xs) < 1e-6
+        if taps > 1:
+            assert rel(st, last) < 1e-6
+    plain, xn, _ = Lr.sandwich_norm_conv(x, w, b, 1e-5, cw, garbage.copy(), 0)          # nothing owed: the stream stays as it is
+    assert np.array_equal(xn, x) and rel(plain, O.conv_added(O.layer_norm(t64(x), t64(w), t64(b), 1e-5), t64(cw))[0]) < 1e-6
+
+
 def test_polynomial_activation_and_gated_norm():
     from ntransformer_amd import layers as Lr
     g = np.random.default_rng(5)
@@ -251,8 +283,10 @@ def test_lightning_recurrence_whole_portions_and_single_tokens(dn, dv):
     ref, Sref = _plain_lightning(q, k, v, decay, H, dn, dv)
     whole, S = Lr.lightning_attention(q, k, v, decay, H, dn, dv, 0)
     assert rel(whole, ref) < 1e-5 and rel(S, Sref) < 1e-5
+    turn, S = Lr.lightning_attention(q, k, v, decay, H, dn, dv, 0, side_by_side=False)       # the chunks in turn by one workgroup == side by side
+    assert rel(turn, ref) < 1e-5 and rel(S, Sref) < 1e-5 and rel(turn, whole) < 1e-5
     parts, at, S = [], 0, None
-    for n in [2, 63, 1, 1, 64, 3, 16]:
+    for n in [2, 63, 1, 8, 57, 3, 16]:
         o, S = Lr.lightning_attention(q[at:at + n], k[at:at + n], v[at:at + n], decay, H, dn, dv, at, state=S)
         parts.append(o)
         at += n
@@ -280,6 +314,7 @@ def test_lightning_remembers_a_far_token_and_starts_from_zeros():
     q[T - 1, 0] = 2.0
     out, S = Lr.lightning_attention(q, k, v, [1.0], H, dn, dv, 0, silu=False)
     assert np.abs(out[T - 1] - 6.0 * v[3]).max() < 1e-4
+    assert np.abs(Lr.lightning_attention(q, k, v, [1.0], H, dn, dv, 0, silu=False, side_by_side=False)[0][T - 1] - 6.0 * v[3]).max() < 1e-4
     half, S1 = Lr.lightning_attention(q[:400], k[:400], v[:400], [1.0], H, dn, dv, 0, silu=False)
     rest, _ = Lr.lightning_attention(q[400:], k[400:], v[400:], [1.0], H, dn, dv, 400, state=S1, silu=False)
     assert np.abs(rest[-1] - 6.0 * v[3]).max() < 1e-4
