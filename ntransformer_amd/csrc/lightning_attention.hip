@@ -53,10 +53,18 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(const LightArgs a)
     const float L = a.log_decay[h];
     // kWhole: the sequence's state; kLocal / kOutputs: this chunk's slot of the scratch [chunks][H][dn][dv] (written / read)
     float* sg = (MODE == kWhole ? a.state : a.scratch + (long long)blockIdx.z * a.H * a.dn * a.dv) + ((long long)h * a.dn) * a.dv + v0;
-    for (int e = tid; e < DP * LV; e += 256) {
-        const int d = e / LV, c = e % LV;
-        const bool have = MODE == kOutputs || (MODE == kWhole && a.pos0 > 0);
-        Ss[e] = (have && d < a.dn && c < nv) ? sg[(long long)d * a.dv + c] : 0.0f;
+    // (every staging loop below asks for eight of a thread's entries before it uses the first: a workgroup fills the LDS of its CU, so nobody else hides its latency)
+    const bool have = MODE == kOutputs || (MODE == kWhole && a.pos0 > 0);
+    for (int e0 = tid; e0 < DP * LV; e0 += 256 * 8) {
+        float x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int e = e0 + 256 * u, d = e / LV, c = e % LV;
+            x[u] = (have && e < DP * LV && d < a.dn && c < nv) ? sg[(long long)d * a.dv + c] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (e0 + 256 * u < DP * LV) Ss[e0 + 256 * u] = x[u];
     }
     const int ti = tid / 16, tj = tid % 16;        // 16 x 16 thread grid
     constexpr int RI = C / 16;                     // token rows per thread (C = 64: 4, C = 32: 2)
@@ -66,19 +74,31 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(const LightArgs a)
         const int nr = min(C, (n + RI - 1) / RI * RI);   // rows a thread tile may touch: the chunk's tokens rounded up to whole tiles
         __syncthreads();                           // the last chunk's readers are done (and the state slice is in place)
         if (tid < C) Ws[tid] = tid < n ? decay_pow(L, n - 1 - tid) : 0.0f;
-        for (int e = tid; e < nr * DP; e += 256) {
-            const int i = e / DP, d = e % DP;
-            float qv = 0.0f, kv = 0.0f;
-            if (i < n && d < a.dn) {
-                qv = maybe_silu(a.q[(long long)(t0 + i) * a.ldq + h * a.dn + d], a.silu);
-                kv = maybe_silu(a.k[(long long)(t0 + i) * a.ldk + h * a.dn + d], a.silu);
+        for (int e0 = tid; e0 < nr * DP; e0 += 256 * 8) {
+            float qv[8], kv[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int e = e0 + 256 * u, i = e / DP, d = e % DP;
+                const bool in = e < nr * DP && i < n && d < a.dn;
+                qv[u] = in && MODE != kLocal ? a.q[(long long)(t0 + i) * a.ldq + h * a.dn + d] : 0.0f;     // (the local sums need no queries)
+                kv[u] = in ? a.k[(long long)(t0 + i) * a.ldk + h * a.dn + d] : 0.0f;
             }
-            Qs[i * LQ + d] = qv;
-            Ks[i * LQ + d] = kv;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int e = e0 + 256 * u, i = e / DP, d = e % DP;
+                if (e < nr * DP) { Qs[i * LQ + d] = maybe_silu(qv[u], a.silu); Ks[i * LQ + d] = maybe_silu(kv[u], a.silu); }
+            }
         }
-        for (int e = tid; e < nr * LV; e += 256) {
-            const int i = e / LV, c = e % LV;
-            Vs[e] = (i < n && c < nv) ? maybe_silu(a.v[(long long)(t0 + i) * a.ldv + h * a.dv + v0 + c], a.silu) : 0.0f;
+        for (int e0 = tid; e0 < nr * LV; e0 += 256 * 8) {
+            float x[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int e = e0 + 256 * u, i = e / LV, c = e % LV;
+                x[u] = (e < nr * LV && i < n && c < nv) ? a.v[(long long)(t0 + i) * a.ldv + h * a.dv + v0 + c] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (e0 + 256 * u < nr * LV) Vs[e0 + 256 * u] = maybe_silu(x[u], a.silu);
         }
         __syncthreads();
         // ---- decayed scores inside the chunk: thread (ti, tj) owns tokens i = ti * RI + r against j = tj * RI + c

@@ -97,12 +97,17 @@ __global__ __launch_bounds__(256) void window_attention_kernel(const WinArgs a) 
     const int jlo = a.window > 0 ? max(0, pmin - a.window + 1) : 0;
     const int jhi = pmax;   // inclusive
     // queries into LDS
-    for (int e = threadIdx.x; e < WROWS * M * DNP; e += 256) {
-        const int i = e / (M * DNP), md = e % (M * DNP), m = md / DNP, d = md % DNP;
-        const int rho = row0 + i;
-        float qv = 0.0f;
-        if (rho < n_rows && d < a.dn) qv = a.q[(long long)(rho / R) * a.ldq + ((long long)(g * R + rho % R) * M + m) * a.dn + d];
-        Qs[e] = qv;
+    for (int e0 = threadIdx.x; e0 < WROWS * M * DNP; e0 += 256 * 4) {     // (four of a thread's entries asked for before the first is stored)
+        float qv[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int e = e0 + 256 * u, i = e / (M * DNP), md = e % (M * DNP), m = md / DNP, d = md % DNP;
+            const int rho = row0 + i;
+            qv[u] = (e < WROWS * M * DNP && rho < n_rows && d < a.dn) ? a.q[(long long)(rho / R) * a.ldq + ((long long)(g * R + rho % R) * M + m) * a.dn + d] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (e0 + 256 * u < WROWS * M * DNP) Qs[e0 + 256 * u] = qv[u];
     }
     float mx[M][WQPW], l[M][WQPW], acc[M][WQPW][WMAXC];
     int rpos[WQPW];
