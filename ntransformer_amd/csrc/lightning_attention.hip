@@ -265,11 +265,13 @@ __global__ __launch_bounds__(256) void lightning_step_kernel(const LightArgs a) 
 using namespace ntk;
 
 static int light_chunk(int dn) { return dn > 128 ? 32 : 64; }   // chunk length: the LDS of two [C][dn] chunks, the value slab, the state slice and the scores
+// side by side the chunks are 32 tokens long: half the LDS per workgroup (two of them share a CU and hide each other's round trips), twice the workgroups
+static int light_chunk_parallel(int) { return 32; }
 
 size_t ntk_lightning_attention_scratch(int T, int H, int dn, int dv) {
     if (T <= 0 || H <= 0 || dn <= 0 || dv <= 0) return 0;
-    const int C = light_chunk(dn);
-    return T > C ? (size_t)((T + C - 1) / C) * H * dn * dv : 0;
+    const int C = light_chunk_parallel(dn);
+    return T > light_chunk(dn) ? (size_t)((T + C - 1) / C) * H * dn * dv : 0;
 }
 
 int ntk_lightning_attention(float* out, int ldo, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* log_decay, float* state,
@@ -289,7 +291,8 @@ int ntk_lightning_attention(float* out, int ldo, const float* q, int ldq, const 
         return last_launch_status();
     }
     const int DP = (dn + 15) & ~15;
-    const int C = light_chunk(dn);
+    const bool side = scratch && T > light_chunk(dn);
+    const int C = side ? light_chunk_parallel(dn) : light_chunk(dn);
     const size_t lds = ((size_t)2 * C * (DP + 1) + (size_t)C * LV + (size_t)DP * LV + (size_t)C * (C + 1) + C) * sizeof(float);
     if (lds > 156 * 1024) return NTK_E_SHAPE;
     static bool raised = false;   // (idempotent: a race sets the same attribute twice)
@@ -302,7 +305,7 @@ int ntk_lightning_attention(float* out, int ldo, const float* q, int ldq, const 
         NTK_HIP_TRY(hipFuncSetAttribute((const void*)lightning_chunk_kernel<32, kOutputs>, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
         raised = true;
     }
-    if (!scratch || T <= C) {
+    if (!side) {
         const dim3 grid(H, slabs);
         if (C == 64) hipLaunchKernelGGL((lightning_chunk_kernel<64, kWhole>), grid, dim3(256), lds, s, a);
         else hipLaunchKernelGGL((lightning_chunk_kernel<32, kWhole>), grid, dim3(256), lds, s, a);

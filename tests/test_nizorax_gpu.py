@@ -485,6 +485,8 @@ def test_slots_side_by_side_freed_and_used_again(tmp_path):
          ff=16, eff=16, shared_ff=16, experts=4, top=4, groups=(2, 2), taps=2, decay=0.9, scaling=False),                         # equal sizes, kept groups = all, scalar decay
     dict(layers=("attention", "lightning", "attention"), mlps=("moe", "dense", None), loop=(1, 3, 3), rot_dims=4, width=40, heads=3, kv_heads=3, dim=10,
          vdim=6, lheads=5, ldim=7, lvdim=9, decay=(0.3, 0.7, 0.9, 0.99, 1.0), ff=50, vocab=50, taps=4, experts=9, groups=(3, 1), top=3),  # a layer ahead of the span, odd sizes, a layer without feed-forward
+    dict(layers=("attention", "lightning"), mlps=("moe", "dense"), width=36, vocab=37, heads=2, kv_heads=1, dim=6, vdim=5, rot_dims=2, lheads=2, ldim=9, lvdim=7,
+         decay=(0.8, 0.95), ff=30, eff=10, shared_ff=6, experts=4, groups=(4, 2), top=2, window=3, taps=3),                      # sizes that are multiples of nothing, groups of one expert
     dict(layers=("lightning",), mlps=(None,), taps=5, lheads=1, decay=(0.0,)),                                                     # nothing but a forgetting mixer
     dict(layers=("attention", "lightning"), mlps=("moe", "moe"), width=128, heads=6, kv_heads=2, dim=72, vdim=80, rot_dims=32, lheads=2, ldim=136, lvdim=72,
          decay=(0.95, 0.999), experts=16, top=3, groups=(2, 1), eff=24, shared_ff=40, window=33),                                  # head sizes past one 64-entry slab, the short-chunk form of the recurrence
