@@ -3,7 +3,8 @@
 // A family registers a factory under the "architecture" string of its config.json (a static FamilyRegistrar in its .cpp).  open_model(path) reads
 // that string and builds the object; GGUF files stay with nt::Model (engine/model.h), which the engine holds directly.
 // A SequenceModel owns its weights and a slot cache: every live sequence holds one slot, tokens are appended with forward() in portions of any size,
-// and a released slot is handed to the next sequence as it is (nothing a sequence reads lies beyond its own length).
+// and a released slot is handed to the next sequence as it is (nothing a sequence reads lies beyond its own length; what a slot holds besides rows per
+// position -- a recurrent state, the last inputs of a convolution -- is not read by a sequence's first token).
 #pragma once
 #include <cstdint>
 #include <functional>
@@ -36,7 +37,7 @@ public:
     virtual int acquire_slot() = 0;                 // slot id >= 0 (length 0), or NTK_E_NOMEM when all are taken
     virtual int release_slot(int slot) = 0;
     virtual int slot_length(int slot) const = 0;    // positions the slot holds, negative if it is not live
-    virtual int truncate_slot(int slot, int length) = 0;   // forget everything from position `length` on
+    virtual int truncate_slot(int slot, int length) = 0;   // forget everything from position `length` on (a family with recurrent state: only back to 0 or not at all)
     // ---- the step: append `n` tokens to `slot`; the logits of the tokens want[0 .. n_want) (indices into this portion) are left on the device,
     //      [n_want][vocab] F32, and returned (stream ordered: sync() or copy_logits() before the host reads).  nullptr on failure.
     virtual float* forward(int slot, const int* tokens, int n, const int* want, int n_want) = 0;
@@ -56,8 +57,8 @@ std::vector<std::string> registered_families();
 std::unique_ptr<SequenceModel> make_family(const std::string& architecture);
 std::unique_ptr<SequenceModel> open_model(const std::string& path, const SeqLoadOptions& opt, std::string* why);
 
-// The slot cache: `slots` regions of `capacity` positions; a live slot has a length.  Device memory belongs to the model (one block per layer run,
-// [slots][capacity][row]); this class is the bookkeeping every family shares.
+// The slot cache: `slots` regions of `capacity` positions; a live slot has a length.  Device memory belongs to the model (per layer run: cache rows
+// [slots][capacity][row], and per slot whatever state its mixers carry); this class is the bookkeeping every family shares.
 class SlotTable {
 public:
     void reset(int slots, int capacity) { len_.assign((size_t)slots, -1); cap_ = capacity; }
